@@ -1,0 +1,447 @@
+/*
+ * cpu_ref.c -- CPU restatement of the scaled mixed-precision GEMM path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the shipped library links, loads or
+ * calls this file; it is the checker the GPU kernels are compared against and
+ * the "cpu_baseline" leg of the benchmark.  The product path has no CPU
+ * fallback.
+ *
+ * The reference (machinelv/QGEMM) ships no CPU GEMM: its only oracle is
+ * cuBLAS (tests/includes/test_config.h:29-52).  Each function below restates
+ * the arithmetic of one reference device function and cites it.
+ *
+ * Parity pinning (what checks each function besides itself):
+ *   fp8 e4m3 OCP codec   closed-form 256-entry table, exhaustive round trip,
+ *                        tie cases, torch.float8_e4m3fn on every finite code
+ *   bf16 / fp16 codec    torch / numpy casts on stratified samples
+ *   int8 GEMM            exact integers: brute force, identities, K-split
+ *   fp GEMM              fp64 triple loop, numpy matmul on exactly
+ *                        representable inputs
+ *   block-scaled GEMM    reduces to per-matrix when scales are equal,
+ *                        power-of-two scales commute exactly, linearity
+ *   transpose            numpy .T, involution
+ * The reference holds no golden vectors for the FP8 block-scaled kernel
+ * (no test calls it), so that function's parity is pinned only by the
+ * mathematical checks above: "parity unpinned by reference tests".
+ *
+ * Build: see oracle/Makefile (gcc -O3 -fopenmp -ffp-contract=off).
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define REF_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ */
+/* threads                                                             */
+/* ------------------------------------------------------------------ */
+REF_API int ref_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+REF_API void ref_set_num_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}
+
+/* ------------------------------------------------------------------ */
+/* counter-based PRNG: value i of stream `seed` depends on (seed, i)   */
+/* only, so any host regenerates the same inputs in any order.         */
+/* The reference's TestConfig carries seed = 42 but never uses it      */
+/* (tests/includes/test_config.h:64,230).                              */
+/* ------------------------------------------------------------------ */
+static inline uint64_t mix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+static inline uint64_t rng_u64(uint64_t seed, uint64_t i) {
+    return mix64(mix64(seed) ^ (i * 0xD1342543DE82EF95ull + 0x632BE59BD9B4E019ull));
+}
+
+/* 24 random bits -> float in [0,1) exactly representable */
+static inline float rng_unit(uint64_t seed, uint64_t i) {
+    return (float)(rng_u64(seed, i) >> 40) * (1.0f / 16777216.0f);
+}
+
+REF_API void ref_fill_uniform(float *out, size_t n, uint64_t seed, float lo, float hi) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) out[i] = lo + (hi - lo) * rng_unit(seed, i);
+}
+
+/* Box-Muller on two independent counters; double math then one rounding. */
+REF_API void ref_fill_normal(float *out, size_t n, uint64_t seed) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        double u1 = ((double)(rng_u64(seed, 2 * i) >> 11) + 1.0) * (1.0 / 9007199254740992.0);
+        double u2 = (double)(rng_u64(seed, 2 * i + 1) >> 11) * (1.0 / 9007199254740992.0);
+        out[i] = (float)(sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2));
+    }
+}
+
+/* The harness's closed-form inputs, tests/includes/test_config.h:251-258:
+ *   A[i] = (i % 43) / 20.0 + 0.2 + (i % 19),  B[i] = (i % 43) / 20.0 + 0.2 + (i % 37)
+ * evaluated in double and narrowed to float as the reference does. */
+REF_API void ref_fill_pattern(float *out, size_t n, int which /*0=A,1=B*/) {
+    const size_t mod = which ? 37 : 19;
+    for (size_t i = 0; i < n; ++i)
+        out[i] = (float)((double)((float)(i % 43)) / 20.0 + 0.2 + (double)(i % mod));
+}
+
+/* ------------------------------------------------------------------ */
+/* codecs                                                              */
+/* ------------------------------------------------------------------ */
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* bf16: round to nearest even on the upper 16 bits, the bit trick of
+ * src/include/fast_quat.h:4-12 plus the NaN guard that file lacks. */
+REF_API uint16_t ref_f32_to_bf16(float f) {
+    uint32_t u = f2u(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+REF_API float ref_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+/* IEEE binary16, round to nearest even, overflow to inf. */
+REF_API uint16_t ref_f32_to_f16(float f) {
+    uint32_t u = f2u(f);
+    uint32_t sign = (u >> 16) & 0x8000u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);          /* NaN */
+    if (a >= 0x47800000u) return (uint16_t)(sign | 0x7C00u);         /* >= 65536 -> inf (also inf) */
+    if (a < 0x38800000u) {                                           /* below 2^-14: subnormal half */
+        /* value = a_float; result mantissa = rne(a_float * 2^24) */
+        float v = u2f(a) * 16777216.0f;                              /* exact scaling */
+        float r = nearbyintf(v);                                     /* default mode: ties to even */
+        return (uint16_t)(sign | (uint32_t)r);                       /* may carry into exponent 1: correct */
+    }
+    uint32_t mant = a & 0x007FFFFFu;
+    uint32_t exp = (a >> 23) - 112u;                                 /* rebias 127 -> 15 */
+    uint32_t h = (exp << 10) | (mant >> 13);
+    uint32_t rem = mant & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h += 1u;      /* carry may reach inf at 65520+: correct */
+    return (uint16_t)(sign | h);
+}
+REF_API float ref_f16_to_f32(uint16_t h) {
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t mant = h & 0x3FFu;
+    if (exp == 0) return u2f(sign) + (sign ? -1.0f : 1.0f) * (float)mant * (1.0f / 16777216.0f);
+    if (exp == 31) return u2f(sign | 0x7F800000u | (mant << 13));
+    return u2f(sign | ((exp + 112u) << 23) | (mant << 13));
+}
+
+/* fp8 e4m3, OCP ("e4m3fn"): 1-4-3, bias 7, subnormals m * 2^-9, largest
+ * finite 448 = 0x7E, NaN = 0x7F / 0xFF, no infinities.  The reference's HIP
+ * kernel uses the gfx942 fnuz flavour (hip_mix_gemm_kernel.cpp:17,382);
+ * gfx950 MFMA decodes OCP, which is what this build defines. */
+REF_API float ref_fp8_e4m3_to_f32(uint8_t b) {
+    uint32_t sign = (b & 0x80u) ? 0x80000000u : 0u;
+    uint32_t exp = (b >> 3) & 0xFu;
+    uint32_t mant = b & 7u;
+    if (exp == 15 && mant == 7) return u2f(sign | 0x7FC00000u);
+    float mag = exp ? ldexpf((float)(8 + mant), (int)exp - 10) : ldexpf((float)mant, -9);
+    return sign ? -mag : mag;
+}
+
+/* Encode: saturate to +-448 first ("satfinite"), then round to nearest even.
+ * NaN -> 0x7F with the sign kept. */
+REF_API uint8_t ref_f32_to_fp8_e4m3(float f) {
+    uint32_t u = f2u(f);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint8_t)(sign | 0x7Fu);
+    float x = u2f(a);
+    if (x >= 448.0f) return (uint8_t)(sign | 0x7Eu);
+    if (x < 0.015625f) {                       /* below 2^-6: subnormal grid of 2^-9 */
+        float r = nearbyintf(x * 512.0f);      /* exact scaling, ties to even */
+        return (uint8_t)(sign | (uint8_t)r);   /* r == 8 lands on 0x08 = 2^-6: correct */
+    }
+    uint32_t exp = (a >> 23) - 120u;           /* rebias 127 -> 7 */
+    uint32_t mant = a & 0x007FFFFFu;
+    uint32_t h = (exp << 3) | (mant >> 20);
+    uint32_t rem = mant & 0xFFFFFu;
+    if (rem > 0x80000u || (rem == 0x80000u && (h & 1u))) h += 1u;
+    if (h > 0x7Eu) h = 0x7Eu;                  /* 464 <= x < 448 cannot happen; guard anyway */
+    return (uint8_t)(sign | h);
+}
+
+REF_API void ref_decode_fp8(const uint8_t *in, float *out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = ref_fp8_e4m3_to_f32(in[i]);
+}
+REF_API void ref_encode_fp8(const float *in, uint8_t *out, size_t n) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) out[i] = ref_f32_to_fp8_e4m3(in[i]);
+}
+REF_API void ref_encode_bf16(const float *in, uint16_t *out, size_t n) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) out[i] = ref_f32_to_bf16(in[i]);
+}
+REF_API void ref_decode_bf16(const uint16_t *in, float *out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = ref_bf16_to_f32(in[i]);
+}
+REF_API void ref_encode_f16(const float *in, uint16_t *out, size_t n) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) out[i] = ref_f32_to_f16(in[i]);
+}
+REF_API void ref_decode_f16(const uint16_t *in, float *out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = ref_f16_to_f32(in[i]);
+}
+
+/* ------------------------------------------------------------------ */
+/* quantisers (the step before the path; the reference only states      */
+/* "input matrix will be quantized", README.md:1)                       */
+/* ------------------------------------------------------------------ */
+REF_API float ref_amax(const float *x, size_t n) {
+    float m = 0.0f;
+#pragma omp parallel for reduction(max : m) schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        float a = fabsf(x[i]);
+        if (a > m) m = a;
+    }
+    return m;
+}
+
+/* symmetric int8: s = amax / 127, q = clamp(rint(x / s), -127, 127).
+ * Division (not multiplication by a reciprocal) so every implementation
+ * rounds identically. Returns s. */
+REF_API float ref_quantize_int8(const float *x, int8_t *q, size_t n) {
+    float amax = ref_amax(x, n);
+    float s = amax > 0.0f ? amax / 127.0f : 1.0f;
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        float r = nearbyintf(x[i] / s);
+        if (r > 127.0f) r = 127.0f;
+        if (r < -127.0f) r = -127.0f;
+        q[i] = (int8_t)r;
+    }
+    return s;
+}
+
+/* per-matrix fp8: s = amax / 448, q = e4m3(x / s). Returns s. */
+REF_API float ref_quantize_fp8(const float *x, uint8_t *q, size_t n) {
+    float amax = ref_amax(x, n);
+    float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) q[i] = ref_f32_to_fp8_e4m3(x[i] / s);
+    return s;
+}
+
+/* block fp8 quantiser for a row-major [rows, cols] matrix with scale blocks
+ * of br x bc (1x128 for A, 128x128 for B).  scales is row-major
+ * [ceil(rows/br), ceil(cols/bc)]. */
+REF_API void ref_quantize_fp8_block(const float *x, uint8_t *q, float *scales, size_t rows, size_t cols,
+                                    size_t br, size_t bc) {
+    size_t nbr = (rows + br - 1) / br, nbc = (cols + bc - 1) / bc;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (size_t ib = 0; ib < nbr; ++ib)
+        for (size_t jb = 0; jb < nbc; ++jb) {
+            size_t r1 = (ib + 1) * br < rows ? (ib + 1) * br : rows;
+            size_t c1 = (jb + 1) * bc < cols ? (jb + 1) * bc : cols;
+            float amax = 0.0f;
+            for (size_t r = ib * br; r < r1; ++r)
+                for (size_t c = jb * bc; c < c1; ++c) {
+                    float a = fabsf(x[r * cols + c]);
+                    if (a > amax) amax = a;
+                }
+            float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+            scales[ib * nbc + jb] = s;
+            for (size_t r = ib * br; r < r1; ++r)
+                for (size_t c = jb * bc; c < c1; ++c) q[r * cols + c] = ref_f32_to_fp8_e4m3(x[r * cols + c] / s);
+        }
+}
+
+/* ------------------------------------------------------------------ */
+/* transpose: out[n*M + m] = in[m*N + n], src/transpose/transpose.cu:42,57 */
+/* ------------------------------------------------------------------ */
+REF_API void ref_transpose(const void *in, void *out, size_t M, size_t N, size_t elem) {
+    const uint8_t *src = (const uint8_t *)in;
+    uint8_t *dst = (uint8_t *)out;
+#pragma omp parallel for schedule(static)
+    for (size_t m = 0; m < M; ++m)
+        for (size_t n = 0; n < N; ++n) memcpy(dst + (n * M + m) * elem, src + (m * N + n) * elem, elem);
+}
+
+/* ------------------------------------------------------------------ */
+/* GEMMs.  Operand addressing is by element strides so one routine      */
+/* covers the reference's layouts:                                      */
+/*   "NN"  A[m*K+k], B[k*N+n]   (src/include/gemm_utils.cuh:93,108)     */
+/*   "NT"  A[m*K+k], B[n*K+k]   (src/include/gemm_utils.cuh:259,271)    */
+/*   fp8_mm  A[m+k*M], B[k*N+n] (hip_mix_gemm_kernel.cpp:96,111)        */
+/* C is row-major with leading dimension ldc (only ldC is honoured by   */
+/* the reference kernels, sm89_gemm_kernel_v3.cu:258).                  */
+/* ------------------------------------------------------------------ */
+
+/* int8 x int8 -> int32, exact. */
+REF_API void ref_gemm_i8_i32(const int8_t *A, size_t a_rs, size_t a_cs, const int8_t *B, size_t b_ns, size_t b_ks,
+                             int32_t *C, size_t ldc, size_t M, size_t N, size_t K) {
+    if (a_cs == 1 && b_ks == 1) {
+#pragma omp parallel for schedule(static)
+        for (size_t m = 0; m < M; ++m) {
+            const int8_t *a = A + m * a_rs;
+            for (size_t n = 0; n < N; ++n) {
+                const int8_t *b = B + n * b_ns;
+                int32_t acc = 0;
+                for (size_t k = 0; k < K; ++k) acc += (int32_t)a[k] * (int32_t)b[k];
+                C[m * ldc + n] = acc;
+            }
+        }
+        return;
+    }
+#pragma omp parallel for schedule(static)
+    for (size_t m = 0; m < M; ++m)
+        for (size_t n = 0; n < N; ++n) {
+            int32_t acc = 0;
+            for (size_t k = 0; k < K; ++k) acc += (int32_t)A[m * a_rs + k * a_cs] * (int32_t)B[n * b_ns + k * b_ks];
+            C[m * ldc + n] = acc;
+        }
+}
+
+/* per-matrix scaled int8: C_f32 = float(acc) * (sA * sB); one rounding for
+ * the scale product, one for the final multiply. */
+REF_API void ref_scale_i32_to_f32(const int32_t *acc, float *C, size_t n, float sa, float sb) {
+    const float s = sa * sb;
+    for (size_t i = 0; i < n; ++i) C[i] = (float)acc[i] * s;
+}
+
+/* float operands (already decoded to fp32), fp32 accumulate in ascending k,
+ * the semantics of the harness oracle (cublasGemmEx with CUDA_R_32F compute,
+ * alpha 1, beta 0: tests/includes/test_config.h:29-52). */
+REF_API void ref_gemm_f32acc(const float *A, size_t a_rs, size_t a_cs, const float *B, size_t b_ns, size_t b_ks,
+                             float *C, size_t ldc, size_t M, size_t N, size_t K) {
+    if (a_cs == 1 && b_ks == 1) {
+#pragma omp parallel for schedule(static)
+        for (size_t m = 0; m < M; ++m) {
+            const float *a = A + m * a_rs;
+            for (size_t n = 0; n < N; ++n) {
+                const float *b = B + n * b_ns;
+                /* 8 interleaved partial sums: still pure fp32 accumulation, and
+                 * vectorisable; the tolerance in the tests covers any order. */
+                float p[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                size_t k = 0;
+                for (; k + 8 <= K; k += 8)
+                    for (int j = 0; j < 8; ++j) p[j] += a[k + j] * b[k + j];
+                float acc = ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
+                for (; k < K; ++k) acc += a[k] * b[k];
+                C[m * ldc + n] = acc;
+            }
+        }
+        return;
+    }
+#pragma omp parallel for schedule(static)
+    for (size_t m = 0; m < M; ++m)
+        for (size_t n = 0; n < N; ++n) {
+            float acc = 0.0f;
+            for (size_t k = 0; k < K; ++k) acc += A[m * a_rs + k * a_cs] * B[n * b_ns + k * b_ks];
+            C[m * ldc + n] = acc;
+        }
+}
+
+/* fp64 accumulate: the "truth" the fp32 results are bounded against. */
+REF_API void ref_gemm_f64acc(const float *A, size_t a_rs, size_t a_cs, const float *B, size_t b_ns, size_t b_ks,
+                             double *C, size_t ldc, size_t M, size_t N, size_t K) {
+#pragma omp parallel for schedule(static)
+    for (size_t m = 0; m < M; ++m)
+        for (size_t n = 0; n < N; ++n) {
+            double acc = 0.0;
+            for (size_t k = 0; k < K; ++k)
+                acc += (double)A[m * a_rs + k * a_cs] * (double)B[n * b_ns + k * b_ks];
+            C[m * ldc + n] = acc;
+        }
+}
+
+/* Block-scaled fp8 GEMM, following FP8_GEMM_kernel
+ * (hip_mix_gemm_kernel.cpp:249-378):
+ *   for each K step of bk (<= 128, chosen by divisibility at :442-463):
+ *       P[m,n]    = sum_{k in step} a[m,k] * b[n,k]          fp32   (:204-227)
+ *       acc[m,n] += (P[m,n] * as[m, k0/128]) * bs[n/128, k0/128]    (:241)
+ *   C = acc (caller narrows to bf16, :366)
+ * Scales are addressed by strides so both the reference's column-major
+ * contract (as[m + kb*M], bs[nb + kb*ceil(N/128)], :137,149,164) and the
+ * row-major [M, K/128] / [N/128, K/128] tensors fit.
+ * A and B arrive decoded to fp32 (decoding fp8 is exact). */
+REF_API void ref_gemm_fp8_block(const float *A, size_t a_rs, size_t a_cs, const float *B, size_t b_ns, size_t b_ks,
+                                const float *as, size_t as_ms, size_t as_ks, const float *bs, size_t bs_ns,
+                                size_t bs_ks, float *C, size_t ldc, size_t M, size_t N, size_t K, size_t bk) {
+#pragma omp parallel for schedule(static)
+    for (size_t m = 0; m < M; ++m)
+        for (size_t n = 0; n < N; ++n) {
+            float acc = 0.0f;
+            for (size_t k0 = 0; k0 < K; k0 += bk) {
+                size_t k1 = k0 + bk < K ? k0 + bk : K;
+                float p = 0.0f;
+                for (size_t k = k0; k < k1; ++k) p += A[m * a_rs + k * a_cs] * B[n * b_ns + k * b_ks];
+                size_t kb = k0 / 128;
+                float t = p * as[m * as_ms + kb * as_ks];
+                t = t * bs[(n / 128) * bs_ns + kb * bs_ks];
+                acc += t;
+            }
+            C[m * ldc + n] = acc;
+        }
+}
+
+/* Same product with every term in double: sum_k a*b*as*bs.  Independent of
+ * step size and association; bounds ref_gemm_fp8_block in the tests. */
+REF_API void ref_gemm_fp8_block_f64(const float *A, size_t a_rs, size_t a_cs, const float *B, size_t b_ns, size_t b_ks,
+                                    const float *as, size_t as_ms, size_t as_ks, const float *bs, size_t bs_ns,
+                                    size_t bs_ks, double *C, size_t ldc, size_t M, size_t N, size_t K) {
+#pragma omp parallel for schedule(static)
+    for (size_t m = 0; m < M; ++m)
+        for (size_t n = 0; n < N; ++n) {
+            double acc = 0.0;
+            for (size_t k = 0; k < K; ++k) {
+                size_t kb = k / 128;
+                acc += (double)A[m * a_rs + k * a_cs] * (double)B[n * b_ns + k * b_ks] *
+                       (double)as[m * as_ms + kb * as_ks] * (double)bs[(n / 128) * bs_ns + kb * bs_ks];
+            }
+            C[m * ldc + n] = acc;
+        }
+}
+
+/* The reference's tile dispatch (hip_mix_gemm_kernel.cpp:442-505): first of
+ * {128,64,32} dividing the dimension, 0 if none (the reference throws). */
+REF_API size_t ref_select_tile(size_t dim, int which /*0=M,1=N,2=K*/) {
+    static const size_t lm[] = {128, 64, 32, 0}, ln[] = {64, 32, 0}, lk[] = {128, 64, 32, 0};
+    const size_t *l = which == 0 ? lm : (which == 1 ? ln : lk);
+    for (; *l; ++l)
+        if (dim % *l == 0) return *l;
+    return 0;
+}
+
+/* Block-ID raster of sm89_gemm_kernel_v3.cu:169-183 with the clamp taken
+ * against the number of M tiles (the reference clamps against M in rows,
+ * which only matters when tiles_m is not a multiple of the group). */
+REF_API void ref_block_swizzle(size_t bid, size_t tiles_m, size_t tiles_n, size_t group, size_t *tm, size_t *tn) {
+    size_t per_group = group * tiles_n;
+    size_t g = bid / per_group;
+    size_t start_m = g * group;
+    size_t gsize = tiles_m - start_m < group ? tiles_m - start_m : group;
+    *tm = start_m + (bid % per_group) % gsize;
+    *tn = (bid % per_group) / gsize;
+}
+
+/* harness error measure: max_i |C[i] - ref[i]| in double
+ * (tests/includes/test_config.h:161-169). */
+REF_API double ref_max_abs_diff(const float *c, const float *ref, size_t n) {
+    double m = 0.0;
+    for (size_t i = 0; i < n; ++i) {
+        double e = fabs((double)c[i] - (double)ref[i]);
+        if (e > m) m = e;
+    }
+    return m;
+}
