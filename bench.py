@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Benchmark of the scaled-GEMM hot path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one pass of the hot path over one batch of synthetic input already
+resident in HBM: one fp8-e4m3 per-matrix-scaled GEMM, M = N = K = 8192, fp32
+accumulation, bf16 output (BASELINE.json config 3, the shape the metric is quoted
+on).  Prints ONE JSON line.  `value` is TFLOP/s = 2*M*N*K / time.
+
+Timing protocol: W warm-up launches, then K launches bracketed by
+torch.cuda.synchronize() (wall clock, `ms_per_step`) and by a pair of HIP events
+on the launch stream (`roofline.achieved`): the reference harness's protocol
+(tests/includes/test_config.h:110-135, simple_timer.h:27-41) with its TFLOPS
+formula (:146-147).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published dense peaks
+PEAK_TFLOPS = {"f8": 5000.0, "i8": 5000.0, "bf16": 2500.0, "f16": 2500.0}
+PEAK_HBM_GBS = 8000.0
+
+
+def _time_launches(fn, steps, warmup):
+    """-> (wall ms per step, event ms per launch)"""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, e0.elapsed_time(e1) / steps
+
+
+def _quant_fp8(x):
+    import torch
+    s = (x.abs().max() / 448.0).float().reshape(1)
+    return (x / s).to(torch.float8_e4m3fn), s
+
+
+def _quant_i8(x):
+    import torch
+    s = (x.abs().max() / 127.0).float().reshape(1)
+    return torch.clamp(torch.round(x / s), -127, 127).to(torch.int8), s
+
+
+def cpu_baseline(a_q, b_q, sa, sb, rows):
+    """The CPU oracle (a port: the reference has no CPU GEMM) on the first `rows` rows of C,
+    full N and K, all host cores.  Timed: fp8 decode of the operands + fp32-accumulate GEMM."""
+    import numpy as np
+    from oracle import cpu_ref as R
+    a = a_q[:rows].view(__import__("torch").uint8).cpu().numpy()
+    b = b_q.view(__import__("torch").uint8).cpu().numpy()
+    N, K = b.shape
+    R.gemm_f32acc(R.decode_fp8(a[:8]), R.decode_fp8(b[:64]))       # warm the library and the threads
+    t0 = time.perf_counter()
+    c = R.gemm_f32acc(R.decode_fp8(a), R.decode_fp8(b)) * np.float32(sa * sb)
+    dt = time.perf_counter() - t0
+    return {
+        "value": 2.0 * rows * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": R.num_threads(), "kind": "port",
+        "sample": f"first {rows} rows of C (full N={N}, K={K}) of the same fp8 workload, fp8 decode + fp32-accumulate "
+                  f"GEMM, {dt:.2f} s; extrapolated full problem {dt * (a_q.shape[0] / rows):.0f} s",
+    }, c
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--size", type=int, default=8192, help="M = N = K of the headline workload")
+    ap.add_argument("--cpu-rows", type=int, default=256, help="rows of C the CPU baseline computes (0 = skip)")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists).", file=sys.stderr)
+        return 2
+
+    import torch
+    import qgemm_amd as Q
+    Q.load_library()                      # fails loudly if libqgemm.so is missing: there is no fallback
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.manual_seed(42)                 # seed of the reference harness, tests/includes/test_config.h:64
+    dev = "cuda:0"
+    M = N = K = args.size
+
+    # ---- headline: fp8 per-matrix 8192^3 -> bf16
+    a_q, sa = _quant_fp8(torch.randn(M, K, device=dev))
+    b_q, sb = _quant_fp8(torch.randn(N, K, device=dev))
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    run = lambda: Q.scaled_gemm(a_q, b_q, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)
+    wall_ms, ev_ms = _time_launches(run, args.steps, args.warmup)
+    cfg_name = Q.last_config()
+    flops = 2.0 * M * N * K
+    tflops_wall = flops / (wall_ms * 1e-3) / 1e12
+    tflops_ev = flops / (ev_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "scaled-GEMM TFLOP/s (fp8 e4m3 per-matrix scales, M=N=K=%d), 1 GPU" % M,
+        "value": tflops_wall, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f8e4m3 (fp32 accumulate, bf16 out)", "data": "synthetic",
+        "config": {"workload": f"fp8-e4m3 per-matrix-scaled GEMM M=N=K={M}, A MxK and B NxK K-contiguous, bf16 out",
+                   "kernel": cfg_name},
+        "roofline": {"bound": "mfma", "achieved": tflops_ev, "peak": PEAK_TFLOPS["f8"], "unit": "TFLOP/s",
+                     "frac": tflops_ev / PEAK_TFLOPS["f8"], "traffic": None,
+                     "kernel_ms": ev_ms, "flops_per_launch": flops},
+    }
+
+    # ---- the other configs (short; parity for them is in tests/)
+    if not args.no_extra:
+        extra = {}
+        ai, sai = _quant_i8(torch.randn(M, K, device=dev))
+        bi, sbi = _quant_i8(torch.randn(N, K, device=dev))
+        cf = torch.empty(M, N, dtype=torch.float32, device=dev)
+        _, ms = _time_launches(lambda: Q.int8_mm(ai, bi, sai, sbi, cf), max(5, args.steps // 2), 3)
+        extra["int8_per_matrix_%d" % M] = {"tflops": flops / ms / 1e9, "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["i8"],
+                                           "ms": ms, "kernel": Q.last_config()}
+        del ai, bi, cf
+        # cfg 2: int8 4096^3 -> f32
+        m2 = 4096
+        ai, sai = _quant_i8(torch.randn(m2, m2, device=dev))
+        bi, sbi = _quant_i8(torch.randn(m2, m2, device=dev))
+        cf = torch.empty(m2, m2, dtype=torch.float32, device=dev)
+        _, ms = _time_launches(lambda: Q.int8_mm(ai, bi, sai, sbi, cf), 20, 3)
+        extra["cfg2_int8_4096"] = {"tflops": 2.0 * m2 ** 3 / ms / 1e9, "ms": ms, "kernel": Q.last_config()}
+        # cfg 1: fp16 1024^3, B stored N x K
+        m1 = 1024
+        ah = (torch.rand(m1, m1, device=dev) * 2 - 1).half()
+        bh = (torch.rand(m1, m1, device=dev) * 2 - 1).half()
+        ch = torch.empty(m1, m1, dtype=torch.float16, device=dev)
+        _, ms = _time_launches(lambda: Q.gemm(ah, bh, ch, "nk"), 50, 5)
+        extra["cfg1_fp16_1024"] = {"tflops": 2.0 * m1 ** 3 / ms / 1e9, "ms": ms, "kernel": Q.last_config()}
+        # cfg 4: fp8 block-scaled 6144 x 4608 x 7168
+        m4, n4, k4 = 6144, 4608, 7168
+        a4, _ = _quant_fp8(torch.randn(m4, k4, device=dev))
+        b4, _ = _quant_fp8(torch.randn(n4, k4, device=dev))
+        as4 = torch.rand(m4, k4 // 128, device=dev) * 1.5 + 0.5
+        bs4 = torch.rand(n4 // 128, k4 // 128, device=dev) * 1.5 + 0.5
+        c4 = torch.empty(m4, n4, dtype=torch.bfloat16, device=dev)
+        _, ms = _time_launches(lambda: Q.scaled_gemm(a4, b4, as4, bs4, c4, m4, n4, k4, Q.SCALE_BLOCK128), 20, 3)
+        extra["cfg4_fp8_block_6144x4608x7168"] = {"tflops": 2.0 * m4 * n4 * k4 / ms / 1e9, "ms": ms,
+                                                  "frac_of_peak": 2.0 * m4 * n4 * k4 / ms / 1e9 / PEAK_TFLOPS["f8"],
+                                                  "kernel": Q.last_config()}
+        del a4, b4, c4
+        # cfg 5: skinny split-K, N=7168, K=2048 (bandwidth-bound: report GB/s of algorithmic bytes)
+        n5, k5 = 7168, 2048
+        for m5 in (16, 64, 128):
+            a5, s5a = _quant_fp8(torch.randn(m5, k5, device=dev))
+            # rotate over enough B buffers to exceed the 256 MB Infinity Cache
+            nbuf = 24
+            b5s = [_quant_fp8(torch.randn(n5, k5, device=dev)) for _ in range(nbuf)]
+            c5 = torch.empty(m5, n5, dtype=torch.bfloat16, device=dev)
+            it = [0]
+
+            def run5():
+                bq, sbq = b5s[it[0] % nbuf]
+                it[0] += 1
+                Q.scaled_gemm(a5, bq, s5a, sbq, c5, m5, n5, k5, Q.SCALE_PER_MATRIX)
+            _, ms = _time_launches(run5, 96, 24)
+            nbytes = n5 * k5 + m5 * k5 + m5 * n5 * 2
+            extra["cfg5_fp8_skinny_M%d" % m5] = {
+                "tflops": 2.0 * m5 * n5 * k5 / ms / 1e9, "GBps": nbytes / ms / 1e6,
+                "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS, "ms": ms, "kernel": Q.last_config()}
+            del b5s
+        out["extra"] = extra
+
+    # ---- CPU baseline beside it (bounded sample), and a parity spot check of the timed kernel against it
+    if args.cpu_rows > 0:
+        rows = min(args.cpu_rows, M)
+        base, cref = cpu_baseline(a_q, b_q, float(sa), float(sb), rows)
+        out["cpu_baseline"] = base
+        import numpy as np
+        got = c[:rows].float().cpu().numpy()
+        ok = bool(np.all(np.abs(got - cref) <= 1e-2 + 2e-2 * np.abs(cref)))
+        out["parity_spot_check"] = {"rows": rows, "rtol": 2e-2, "atol": 1e-2, "pass": ok}
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

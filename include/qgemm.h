@@ -1,0 +1,131 @@
+/*
+ * qgemm.h -- C ABI of the MI355X (gfx950) scaled mixed-precision GEMM library.
+ *
+ * Plain pointers and sizes only.  Every data pointer is a DEVICE pointer owned
+ * by the caller; calls enqueue work on a HIP stream and return without
+ * synchronising, like the reference launchers (stream 0, no sync:
+ * src/gemm/sm89_gemm_kernel_v3.cu:289-298).  Every entry returns a
+ * qgemm_status_t; the C++ forwarders in gemm.h / mix_gemm.h turn that back
+ * into the reference's print / throw behaviour.
+ */
+#ifndef QGEMM_H_
+#define QGEMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum qgemm_status {
+    QGEMM_OK = 0,
+    QGEMM_ERR_INVALID_ARG = 1,   /* null pointer, zero size, unknown enum value     */
+    QGEMM_ERR_UNSUPPORTED = 2,   /* dtype / layout combination with no kernel        */
+    QGEMM_ERR_NO_DEVICE = 3,     /* no HIP device visible                            */
+    QGEMM_ERR_LAUNCH = 4,        /* hipLaunchKernel or another HIP call failed       */
+    QGEMM_ERR_ALLOC = 5,         /* workspace allocation failed                      */
+    QGEMM_ERR_NOT_DIVISIBLE_M = 6, /* reference dispatch contract: M % 32 != 0       */
+    QGEMM_ERR_NOT_DIVISIBLE_N = 7, /*                              N % 32 != 0       */
+    QGEMM_ERR_NOT_DIVISIBLE_K = 8, /*                              K % 32 != 0       */
+    QGEMM_ERR_TOO_LARGE = 9      /* a dimension or stride exceeds what kernels index */
+} qgemm_status_t;
+
+typedef enum qgemm_dtype {
+    QGEMM_DT_F32 = 0,
+    QGEMM_DT_BF16 = 1,
+    QGEMM_DT_F16 = 2,
+    QGEMM_DT_I8 = 3,
+    QGEMM_DT_F8E4M3 = 4,        /* OCP e4m3 ("e4m3fn"): the encoding gfx950 MFMA decodes */
+    QGEMM_DT_I32 = 5
+} qgemm_dtype_t;
+
+/* Where B's K index runs.  Replaces the two loader families of the reference:
+ * src/include/gemm_utils.cuh:93,108 (B[k*N+n]) and :259,271 (B[n*K+k]). */
+typedef enum qgemm_layout_b {
+    QGEMM_B_KN = 0,             /* "NN": B is K x N row-major, B[k*ldB + n]  (GEMM_kernel_v1..v5)     */
+    QGEMM_B_NK = 1              /* "NT": B is N x K row-major, B[n*ldB + k]  (GEMM_kernel_v3_1, v4_1) */
+} qgemm_layout_b_t;
+
+typedef enum qgemm_scale_mode {
+    QGEMM_SCALE_PER_MATRIX = 1, /* a_scale, b_scale point at one float each                          */
+    QGEMM_SCALE_BLOCK128 = 2    /* a_scale per (row, 128-wide K block), b_scale per 128x128 block     */
+} qgemm_scale_mode_t;
+
+typedef enum qgemm_layout {
+    /* A[m*K + k], B[n*K + k]; a_scale[m*KB + kb], b_scale[nb*KB + kb]  (KB = ceil(K/128)) */
+    QGEMM_LAYOUT_K_CONTIGUOUS = 0,
+    /* The contract of fp8_mm (src/mix_gemm/hip_mix_gemm_kernel.cpp:425-439):
+     * A[m + k*M], B[k*N + n]; a_scale[m + kb*M], b_scale[nb + kb*ceil(N/128)] */
+    QGEMM_LAYOUT_REFERENCE = 1
+} qgemm_layout_t;
+
+/* Library set-up.  Replaces blas::blas_init / blas::blas_destroy
+ * (include/blas.h:33-48): selects the current HIP device, loads the kernels.
+ * Idempotent; the compute entries call it lazily.  qgemm_shutdown frees the
+ * per-device workspace. */
+int qgemm_init(void);
+int qgemm_shutdown(void);
+
+/* Number of visible HIP devices (0 when none): lets a host-only caller decide
+ * without touching any compute entry. */
+int qgemm_device_count(void);
+
+const char *qgemm_status_string(int status);
+
+/* Plain GEMM, C[M,N] = A[M,K] * B, fp32 accumulation (int32 for int8).
+ * Replaces GEMM_kernel_v1 .. v5, v3_1, v4_1 (include/gemm.h:25-66).
+ *   in_dtype   BF16 | F16 | I8 | F8E4M3        out_dtype  F32 | BF16 | F16 (I32 for I8 input)
+ *   A          row-major M x K, leading dimension ldA (elements)
+ *   B          per layout_b, leading dimension ldB (elements)
+ *   C          row-major M x N, leading dimension ldC (elements)
+ *   stream     hipStream_t, NULL = default stream
+ * The reference accepts ldA/ldB and ignores them (its loaders index with K and
+ * N); this entry honours them, which is the same thing for ldA = K, ldB = N|K. */
+int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const void *A, size_t ldA, const void *B, size_t ldB,
+               void *C, size_t ldC, size_t M, size_t N, size_t K, void *stream);
+
+/* Scaled GEMM, C = (A o Q_A) x (B o Q_B).
+ * Replaces select_BLOCK_TILE_SIZE_M / fp8_mm (src/mix_gemm/hip_mix_gemm_kernel.cpp:489-516)
+ * and the int8_mm stub (src/gemm/sm80_gemm_kernel.cu:14-22).
+ *   in_dtype   I8 (int32 accumulate, exact) | F8E4M3 (fp32 accumulate)
+ *   out_dtype  F32 | BF16 | F16 ; I32 with I8 input returns the raw accumulators (scales ignored)
+ *   scale_mode PER_MATRIX: C = acc * (a_scale[0] * b_scale[0])
+ *              BLOCK128  : acc += (P_kb * a_scale[m,kb]) * b_scale[n/128,kb] per 128-wide K block
+ *   layout     see qgemm_layout_t;  C is row-major with leading dimension ldC
+ *   split_k    0 = choose, 1 = never split, n > 1 = split K into n slices (deterministic
+ *              two-pass reduction through the library workspace)
+ * QGEMM_LAYOUT_REFERENCE enforces the reference's dispatch contract and
+ * returns QGEMM_ERR_NOT_DIVISIBLE_{M,N,K} where the reference throws. */
+int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
+                      const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N,
+                      size_t K, int split_k, void *stream);
+
+/* out[n*M + m] = in[m*N + n] for 1-, 2- or 4-byte elements.
+ * Replaces matrix_transpose<T> (src/transpose/transpose.cu:60-74), which
+ * handles 2-byte elements with M % 64 == 0 and N % 32 == 0 only; any M, N here. */
+int qgemm_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t N, void *stream);
+
+/* Tile raster used by the GEMM kernels: linear workgroup id -> (tile_m, tile_n).
+ * Replaces the GROUP_SIZE_M swizzle of src/gemm/sm89_gemm_kernel_v3.cu:169-183
+ * (and fixes its clamp), composed with the 8-XCD remap the reference only names
+ * (XCD_SWIZZLE, include/gpu_type.h:24).  Host-callable so tests can check it is
+ * a bijection. */
+int qgemm_tile_map(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n, uint32_t group_m, uint32_t *tile_m,
+                   uint32_t *tile_n);
+
+/* Tuning / diagnostics (no reference counterpart).
+ * qgemm_set_option("force_config", i) pins tile configuration i (-1 = heuristic);
+ * qgemm_last_config writes the name of the kernel variant the last GEMM call chose. */
+int qgemm_set_option(const char *key, long value);
+int qgemm_last_config(char *buf, size_t buflen);
+
+/* Self-check of the MFMA / LDS-DMA lane layouts the kernels assume, run on the
+ * current device.  Writes a short report into buf; returns QGEMM_OK when every
+ * assumption holds.  (Counterpart of the reference's playground/ layout probes.) */
+int qgemm_selftest_layouts(char *buf, size_t buflen);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QGEMM_H_ */

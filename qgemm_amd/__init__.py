@@ -1,0 +1,13 @@
+"""qgemm_amd -- MI355X (gfx950) scaled mixed-precision GEMM.
+
+The product is the C-ABI library qgemm_amd/libqgemm.so (HIP kernels, declared
+in include/qgemm.h).  This package is the thin Python host side over that ABI:
+torch is used for device memory and streams only.
+"""
+from .lib import QgemmError, load_library, library_path  # noqa: F401
+from .ops import (  # noqa: F401
+    DT_BF16, DT_F16, DT_F32, DT_F8E4M3, DT_I8, DT_I32,
+    LAYOUT_K_CONTIGUOUS, LAYOUT_REFERENCE, SCALE_BLOCK128, SCALE_PER_MATRIX,
+    bf16_mm, fp8_mm, gemm, int8_mm, last_config, matrix_transpose, scaled_gemm, selftest_layouts,
+    set_option, tile_map,
+)

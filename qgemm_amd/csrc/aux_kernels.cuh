@@ -1,0 +1,163 @@
+// Kernels around the MFMA GEMM: the any-shape strided GEMM, the transpose, the
+// split-K reduction.
+#pragma once
+#include "common.h"
+
+namespace qgemm {
+
+// ---------------------------------------------------------------------------
+// element decode (software; used only by the any-shape kernel)
+// ---------------------------------------------------------------------------
+__device__ inline float decode_fp8_e4m3(uint8_t b) {
+    // OCP e4m3: 1-4-3, bias 7, subnormals m * 2^-9, 0x7F / 0xFF NaN
+    const uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+    const uint32_t exp = (b >> 3) & 0xFu, mant = b & 7u;
+    float mag;
+    if (exp == 0) mag = (float)mant * 0.001953125f;
+    else if (exp == 15 && mant == 7) mag = __builtin_nanf("");
+    else mag = __builtin_bit_cast(float, ((exp + 120u) << 23) | (mant << 20));
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, mag) | sign);
+}
+
+template <int IN_DT>
+__device__ inline float load_elem(const void *p, size_t i) {
+    if constexpr (IN_DT == QGEMM_DT_F8E4M3) return decode_fp8_e4m3(((const uint8_t *)p)[i]);
+    else if constexpr (IN_DT == QGEMM_DT_I8) return (float)((const int8_t *)p)[i];
+    else if constexpr (IN_DT == QGEMM_DT_BF16)
+        return __builtin_bit_cast(float, (uint32_t)((const uint16_t *)p)[i] << 16);
+    else return (float)((const _Float16 *)p)[i];
+}
+
+__device__ inline void store_out(void *C, size_t idx, float v, int out_dtype) {
+    if (out_dtype == QGEMM_DT_F32) ((float *)C)[idx] = v;
+    else if (out_dtype == QGEMM_DT_BF16) ((unsigned short *)C)[idx] = f32_to_bf16_bits(v);
+    else ((unsigned short *)C)[idx] = f32_to_f16_bits(v);
+}
+
+// ---------------------------------------------------------------------------
+// Any-shape, any-stride GEMM: one thread per C element.  Carries the shapes the
+// MFMA kernel does not take (K not a multiple of 128 bytes).  Same arithmetic
+// contract: int32 accumulation for int8, fp32 otherwise; block scales folded in
+// per `bk` K elements as (P * as) * bs  (hip_mix_gemm_kernel.cpp:231-244).
+// ---------------------------------------------------------------------------
+struct StridedArgs {
+    const void *A, *B;
+    void *C;
+    const float *as, *bs;
+    uint32_t M, N, K;
+    uint64_t a_rs, a_cs, b_ns, b_ks;  // element strides
+    uint64_t ldc;
+    uint32_t as_ms, as_ks, bs_ns, bs_ks;
+    uint32_t bk;                      // K elements per partial product in block mode
+    int out_dtype, scale_mode;        // scale_mode: 0 none, 1 per matrix, 2 block
+};
+
+template <int IN_DT>
+__global__ void __launch_bounds__(256) gemm_strided_kernel(const StridedArgs p) {
+    const uint32_t n = blockIdx.x * 16 + (threadIdx.x & 15);
+    const uint32_t m = blockIdx.y * 16 + (threadIdx.x >> 4);
+    if (m >= p.M || n >= p.N) return;
+    const size_t idx = (size_t)m * p.ldc + n;
+    if constexpr (IN_DT == QGEMM_DT_I8) {
+        int acc = 0;
+        const int8_t *a = (const int8_t *)p.A + (size_t)m * p.a_rs;
+        const int8_t *b = (const int8_t *)p.B + (size_t)n * p.b_ns;
+        for (uint32_t k = 0; k < p.K; ++k) acc += (int)a[k * p.a_cs] * (int)b[k * p.b_ks];
+        if (p.out_dtype == QGEMM_DT_I32) {
+            ((int *)p.C)[idx] = acc;
+            return;
+        }
+        const float s = p.scale_mode == 1 ? p.as[0] * p.bs[0] : 1.0f;
+        store_out(p.C, idx, (float)acc * s, p.out_dtype);
+        return;
+    }
+    float acc = 0.0f;
+    if (p.scale_mode == 2) {
+        for (uint32_t k0 = 0; k0 < p.K; k0 += p.bk) {
+            const uint32_t k1 = k0 + p.bk < p.K ? k0 + p.bk : p.K;
+            float part = 0.0f;
+            for (uint32_t k = k0; k < k1; ++k)
+                part += load_elem<IN_DT>(p.A, (size_t)m * p.a_rs + k * p.a_cs) *
+                        load_elem<IN_DT>(p.B, (size_t)n * p.b_ns + k * p.b_ks);
+            const uint32_t kb = k0 / kScaleBlock;
+            acc += (part * p.as[m * p.as_ms + kb * p.as_ks]) * p.bs[(n / kScaleBlock) * p.bs_ns + kb * p.bs_ks];
+        }
+        store_out(p.C, idx, acc, p.out_dtype);
+        return;
+    }
+    for (uint32_t k = 0; k < p.K; ++k)
+        acc += load_elem<IN_DT>(p.A, (size_t)m * p.a_rs + k * p.a_cs) *
+               load_elem<IN_DT>(p.B, (size_t)n * p.b_ns + k * p.b_ks);
+    const float s = p.scale_mode == 1 ? p.as[0] * p.bs[0] : 1.0f;
+    store_out(p.C, idx, acc * s, p.out_dtype);
+}
+
+// ---------------------------------------------------------------------------
+// Transpose: out[n*M + m] = in[m*N + n]   (src/transpose/transpose.cu:11-58).
+// 64 x 64 element tile through LDS, 256 threads.  The LDS tile is stored with
+// its 4-byte words XOR-swizzled by the row, so both the row-wise fill and the
+// column-wise drain touch 32 distinct banks; no padding column.  Any M, N.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) transpose_kernel(const T *__restrict__ in, T *__restrict__ out, uint32_t M,
+                                                        uint32_t N) {
+    constexpr int TILE = 64;
+    __shared__ T tile[TILE][TILE];
+    const uint32_t m0 = blockIdx.y * TILE, n0 = blockIdx.x * TILE;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;   // 64 x 4
+    constexpr int PER_WORD = sizeof(T) >= 4 ? 1 : 4 / sizeof(T);
+#pragma unroll
+    for (int r = ty; r < TILE; r += 4) {
+        const uint32_t m = m0 + r, n = n0 + tx;
+        if (m < M && n < N) {
+            const int word = (tx / PER_WORD) ^ (r & (TILE / PER_WORD - 1));
+            tile[r][word * PER_WORD + tx % PER_WORD] = in[(size_t)m * N + n];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = ty; r < TILE; r += 4) {
+        const uint32_t n = n0 + r, m = m0 + tx;   // output row n, column m
+        if (n < N && m < M) {
+            const int word = (r / PER_WORD) ^ (tx & (TILE / PER_WORD - 1));
+            out[(size_t)n * M + m] = tile[tx][word * PER_WORD + r % PER_WORD];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Split-K second pass: C[m,n] = cast(scale * sum_z part[z][m,n]), z ascending
+// (a fixed order, so results do not depend on scheduling; int32 stays exact).
+// ---------------------------------------------------------------------------
+struct ReduceArgs {
+    const void *part;      // [nsplit][M][N] f32 or i32
+    void *C;
+    const float *as, *bs;
+    uint32_t M, N, nsplit;
+    uint64_t ldc, plane;   // plane = M*N elements
+    int part_is_i32, out_dtype, per_matrix_scale;
+};
+
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const ReduceArgs p) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= p.plane) return;
+    const uint32_t m = (uint32_t)(i / p.N), n = (uint32_t)(i % p.N);
+    const size_t idx = (size_t)m * p.ldc + n;
+    if (p.part_is_i32) {
+        int acc = 0;
+        for (uint32_t z = 0; z < p.nsplit; ++z) acc += ((const int *)p.part)[z * p.plane + i];
+        if (p.out_dtype == QGEMM_DT_I32) {
+            ((int *)p.C)[idx] = acc;
+            return;
+        }
+        const float s = p.per_matrix_scale ? p.as[0] * p.bs[0] : 1.0f;
+        store_out(p.C, idx, (float)acc * s, p.out_dtype);
+        return;
+    }
+    float acc = 0.0f;
+    for (uint32_t z = 0; z < p.nsplit; ++z) acc += ((const float *)p.part)[z * p.plane + i];
+    const float s = p.per_matrix_scale ? p.as[0] * p.bs[0] : 1.0f;
+    store_out(p.C, idx, acc * s, p.out_dtype);
+}
+
+}  // namespace qgemm

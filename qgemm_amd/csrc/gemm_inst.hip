@@ -1,0 +1,48 @@
+// Instantiates the MFMA GEMM template for one arithmetic family.  Compiled once
+// per family with -DINST_ARITH=<Arith> -DINST_BLOCK=<0|1> -DINST_FN=<table fn>,
+// so the families build in parallel.
+#include "variants.h"
+
+#ifndef INST_ARITH
+#error "compile with -DINST_ARITH=... -DINST_BLOCK=... -DINST_FN=..."
+#endif
+
+namespace qgemm {
+
+template <class C>
+static hipError_t launch_variant(const GemmArgs &a, uint32_t grid, hipStream_t s) {
+    static bool attr_done = false;
+    if (!attr_done) {
+        // more than 64 KiB of dynamic LDS has to be asked for explicitly
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_nt_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(gemm_nt_kernel<C>, dim3(grid), dim3(C::THREADS), C::LDS_BYTES, s, a);
+    return hipGetLastError();
+}
+
+#define ROW(NAME, BM, BN, WM_, WN_, LD)                                                                           \
+    {NAME, INST_ARITH, (bool)INST_BLOCK, BM, BN, GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD>::THREADS, \
+     GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD>::LDS_BYTES, LD,                                   \
+     &launch_variant<GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD>>}
+
+static const Variant kTable[] = {
+    ROW("256x256_w2x4_dma", 256, 256, 2, 4, LOAD_DMA),
+    ROW("256x128_w2x2_dma", 256, 128, 2, 2, LOAD_DMA),
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA),
+    ROW("64x128_w1x4_dma", 64, 128, 1, 4, LOAD_DMA),
+    ROW("32x128_w1x4_dma", 32, 128, 1, 4, LOAD_DMA),
+    ROW("16x128_w1x2_dma", 16, 128, 1, 2, LOAD_DMA),
+    ROW("256x256_w2x4_vgpr", 256, 256, 2, 4, LOAD_VGPR),
+    ROW("128x128_w2x2_vgpr", 128, 128, 2, 2, LOAD_VGPR),
+    ROW("32x128_w1x4_vgpr", 32, 128, 1, 4, LOAD_VGPR),
+};
+
+const Variant *INST_FN(int *count) {
+    *count = (int)(sizeof(kTable) / sizeof(kTable[0]));
+    return kTable;
+}
+
+}  // namespace qgemm

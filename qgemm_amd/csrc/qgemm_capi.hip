@@ -1,0 +1,726 @@
+// extern "C" layer of the library: argument checks, kernel choice, workspace,
+// launches.  Declarations and the reference interfaces they replace are in
+// include/qgemm.h.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "aux_kernels.cuh"
+#include "selftest.cuh"
+#include "variants.h"
+
+using namespace qgemm;
+
+#define QGEMM_EXPORT __attribute__((visibility("default")))
+
+namespace {
+
+struct Context {
+    std::mutex mu;
+    bool ready = false;
+    int device = -1;
+    int num_cus = 256;
+    void *workspace = nullptr;
+    size_t workspace_bytes = 0;
+    long force_config = -1;     // index into the variant table, -1 = heuristic
+    long force_split = 0;       // 0 = heuristic
+    long force_group_m = 0;     // 0 = default
+    std::string last_config;
+};
+
+Context g_ctx;
+
+#define HIP_TRY(expr)                                  \
+    do {                                               \
+        hipError_t e_ = (expr);                        \
+        if (e_ != hipSuccess) return QGEMM_ERR_LAUNCH; \
+    } while (0)
+
+int ensure_init_locked() {
+    if (g_ctx.ready) return QGEMM_OK;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return QGEMM_ERR_NO_DEVICE;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    g_ctx.device = dev;
+    g_ctx.num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    g_ctx.ready = true;
+    return QGEMM_OK;
+}
+
+// Grows the per-process workspace (split-K partial planes, transposed operands).
+// Calls that use it are ordered by the stream they are enqueued on; concurrent
+// calls on different streams would share it and must not overlap.
+int ensure_workspace_locked(size_t bytes, void **out) {
+    if (bytes > g_ctx.workspace_bytes) {
+        if (g_ctx.workspace) {
+            HIP_TRY(hipDeviceSynchronize());
+            HIP_TRY(hipFree(g_ctx.workspace));
+            g_ctx.workspace = nullptr;
+            g_ctx.workspace_bytes = 0;
+        }
+        size_t want = std::max(bytes, (size_t)64 << 20);
+        void *p = nullptr;
+        if (hipMalloc(&p, want) != hipSuccess) return QGEMM_ERR_ALLOC;
+        g_ctx.workspace = p;
+        g_ctx.workspace_bytes = want;
+    }
+    *out = g_ctx.workspace;
+    return QGEMM_OK;
+}
+
+const Variant *table_for(int arith, bool block, int *count) {
+    if (block) return arith == AR_F8 ? variants_f8_block(count) : nullptr;
+    switch (arith) {
+        case AR_I8: return variants_i8(count);
+        case AR_F8: return variants_f8(count);
+        case AR_BF16: return variants_bf16(count);
+        case AR_F16: return variants_f16(count);
+    }
+    return nullptr;
+}
+
+int arith_of(int in_dtype) {
+    switch (in_dtype) {
+        case QGEMM_DT_I8: return AR_I8;
+        case QGEMM_DT_F8E4M3: return AR_F8;
+        case QGEMM_DT_BF16: return AR_BF16;
+        case QGEMM_DT_F16: return AR_F16;
+    }
+    return -1;
+}
+
+bool out_dtype_ok(int in_dtype, int out_dtype) {
+    if (out_dtype == QGEMM_DT_F32 || out_dtype == QGEMM_DT_BF16 || out_dtype == QGEMM_DT_F16) return true;
+    return out_dtype == QGEMM_DT_I32 && in_dtype == QGEMM_DT_I8;
+}
+
+struct NtProblem {
+    int arith;
+    bool block;
+    const void *A, *B;
+    void *C;
+    size_t lda_bytes, ldb_bytes, ldc;   // ldc in elements
+    size_t M, N, Kbytes;
+    const float *as, *bs;
+    uint32_t as_ms, as_ks, bs_ns, bs_ks;
+    int out_dtype, per_matrix, split_k;
+};
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+// Shapes the MFMA kernel takes (pointer alignment is checked separately);
+// everything else goes to the any-shape kernel.
+bool mfma_shape_ok(const NtProblem &q) {
+    return q.Kbytes % 128 == 0 && q.Kbytes > 0 && q.lda_bytes % 16 == 0 && q.ldb_bytes % 16 == 0 &&
+           q.lda_bytes * 256 < ((size_t)1 << 32) && q.ldb_bytes * 256 < ((size_t)1 << 32) &&
+           q.M < ((size_t)1 << 31) && q.N < ((size_t)1 << 31) && q.ldc < ((size_t)1 << 32);
+}
+
+// Heuristic.  Pass 1: the largest tile that still gives every CU a workgroup.
+// Pass 2 (small problems): the shortest tile that covers min(M, 128) rows, so B
+// is streamed once, and the K split below supplies the parallelism.
+int choose_variant(const Variant *tab, int count, size_t M, size_t N, int cus) {
+    const size_t m16 = std::max<size_t>(16, (M + 15) / 16 * 16);
+    for (int i = 0; i < count; ++i) {
+        if (tab[i].loader != LOAD_DMA || (size_t)tab[i].bm > m16) continue;
+        const size_t tiles = ((M + tab[i].bm - 1) / tab[i].bm) * ((N + tab[i].bn - 1) / tab[i].bn);
+        if (tiles >= (size_t)cus) return i;
+    }
+    const size_t target = std::min<size_t>(m16, 128);
+    int best = -1;
+    for (int i = 0; i < count; ++i) {
+        if (tab[i].loader != LOAD_DMA || (size_t)tab[i].bm < target) continue;
+        if (best < 0 || tab[i].bm < tab[best].bm) best = i;
+    }
+    return best;
+}
+
+struct Plan {
+    const Variant *v = nullptr;
+    GemmArgs a;
+    size_t tiles = 0;
+    size_t split_bytes = 0;   // workspace the K split needs (0 when not split)
+};
+
+int plan_nt(const NtProblem &q, Plan &pl) {
+    int count = 0;
+    const Variant *tab = table_for(q.arith, q.block, &count);
+    if (!tab) return QGEMM_ERR_UNSUPPORTED;
+    int vi = g_ctx.force_config >= 0 && g_ctx.force_config < count ? (int)g_ctx.force_config
+                                                                    : choose_variant(tab, count, q.M, q.N, g_ctx.num_cus);
+    if (vi < 0) return QGEMM_ERR_UNSUPPORTED;
+    const Variant &v = tab[vi];
+    pl.v = &v;
+    GemmArgs &a = pl.a;
+    std::memset(&a, 0, sizeof(a));
+    a.as = q.as;
+    a.bs = q.bs;
+    a.M = (uint32_t)q.M;
+    a.N = (uint32_t)q.N;
+    a.ksteps = (uint32_t)(q.Kbytes / 128);
+    a.lda = (uint32_t)q.lda_bytes;
+    a.ldb = (uint32_t)q.ldb_bytes;
+    a.tiles_m = (uint32_t)((q.M + v.bm - 1) / v.bm);
+    a.tiles_n = (uint32_t)((q.N + v.bn - 1) / v.bn);
+    a.group_m = g_ctx.force_group_m > 0 ? (uint32_t)g_ctx.force_group_m : 8;
+    a.as_ms = q.as_ms;
+    a.as_ks = q.as_ks;
+    a.bs_ns = q.bs_ns;
+    a.bs_ks = q.bs_ks;
+    a.nb_max = (uint32_t)((q.N + 127) / 128 - 1);
+    pl.tiles = (size_t)a.tiles_m * a.tiles_n;
+    if (pl.tiles * 64 >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
+
+    uint32_t nsplit = 1;
+    if (q.split_k > 1) nsplit = (uint32_t)q.split_k;
+    else if (q.split_k == 0) {
+        if (g_ctx.force_split > 0) nsplit = (uint32_t)g_ctx.force_split;
+        else if (pl.tiles * 2 <= (size_t)g_ctx.num_cus && a.ksteps >= 8) {
+            // enough slices to cover the CUs about twice, at least 4 K steps each
+            uint32_t want = (uint32_t)((2 * (size_t)g_ctx.num_cus + pl.tiles - 1) / pl.tiles);
+            nsplit = std::min<uint32_t>(want, a.ksteps / 4);
+        }
+    }
+    nsplit = std::max<uint32_t>(1, std::min<uint32_t>(nsplit, a.ksteps));
+    a.ksteps_per_split = (a.ksteps + nsplit - 1) / nsplit;
+    nsplit = (a.ksteps + a.ksteps_per_split - 1) / a.ksteps_per_split;   // no empty slices
+    a.nsplit = nsplit;
+    pl.split_bytes = nsplit > 1 ? q.M * q.N * 4 * (size_t)nsplit : 0;
+    return QGEMM_OK;
+}
+
+// split_ws: workspace of pl.split_bytes (ignored when the plan does not split)
+int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
+    const Variant &v = *pl.v;
+    GemmArgs &a = pl.a;
+    a.A = (const char *)q.A;
+    a.B = (const char *)q.B;
+    const bool i32_acc = q.arith == AR_I8;
+    if (a.nsplit == 1) {
+        a.C = (char *)q.C;
+        a.ldc = (uint32_t)q.ldc;
+        a.out_dtype = q.out_dtype;
+        a.per_matrix_scale = q.per_matrix;
+        const int ob = dtype_bytes(q.out_dtype);
+        const int vec = ob == 4 ? 16 : 8;
+        a.vec_store = ((uintptr_t)q.C % vec == 0) && ((q.ldc * ob) % vec == 0);
+        hipError_t e = v.launch(a, (uint32_t)pl.tiles, stream);
+        g_ctx.last_config = v.name;
+        return e == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
+    }
+
+    // split-K: raw accumulators to the workspace, then one ordered reduction
+    const size_t plane = q.M * q.N;
+    a.C = (char *)split_ws;
+    a.ldc = (uint32_t)q.N;
+    a.split_stride = plane;
+    a.out_dtype = i32_acc ? QGEMM_DT_I32 : QGEMM_DT_F32;
+    a.per_matrix_scale = 0;
+    a.vec_store = (q.N % 4 == 0);
+    hipError_t e = v.launch(a, (uint32_t)(pl.tiles * a.nsplit), stream);
+    if (e != hipSuccess) return QGEMM_ERR_LAUNCH;
+
+    ReduceArgs r;
+    std::memset(&r, 0, sizeof(r));
+    r.part = split_ws;
+    r.C = q.C;
+    r.as = q.as;
+    r.bs = q.bs;
+    r.M = (uint32_t)q.M;
+    r.N = (uint32_t)q.N;
+    r.nsplit = a.nsplit;
+    r.ldc = q.ldc;
+    r.plane = plane;
+    r.part_is_i32 = i32_acc;
+    r.out_dtype = q.out_dtype;
+    r.per_matrix_scale = q.per_matrix;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((plane + 255) / 256)), dim3(256), 0, stream, r);
+    g_ctx.last_config = std::string(v.name) + "_splitk" + std::to_string(a.nsplit);
+    return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
+}
+
+// plan, get the split workspace (plus `extra` bytes behind it for transposed operands), run
+int launch_nt(const NtProblem &q, hipStream_t stream) {
+    Plan pl;
+    int st = plan_nt(q, pl);
+    if (st != QGEMM_OK) return st;
+    void *ws = nullptr;
+    if (pl.split_bytes) {
+        st = ensure_workspace_locked(pl.split_bytes, &ws);
+        if (st != QGEMM_OK) return st;
+    }
+    return run_nt(q, pl, ws, stream);
+}
+
+template <int DT>
+int launch_strided_t(const StridedArgs &s, hipStream_t stream) {
+    dim3 grid((s.N + 15) / 16, (s.M + 15) / 16);
+    hipLaunchKernelGGL(gemm_strided_kernel<DT>, grid, dim3(256), 0, stream, s);
+    return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
+}
+
+int launch_strided(int in_dtype, const StridedArgs &s, hipStream_t stream) {
+    g_ctx.last_config = "strided_any_shape";
+    switch (in_dtype) {
+        case QGEMM_DT_I8: return launch_strided_t<QGEMM_DT_I8>(s, stream);
+        case QGEMM_DT_F8E4M3: return launch_strided_t<QGEMM_DT_F8E4M3>(s, stream);
+        case QGEMM_DT_BF16: return launch_strided_t<QGEMM_DT_BF16>(s, stream);
+        case QGEMM_DT_F16: return launch_strided_t<QGEMM_DT_F16>(s, stream);
+    }
+    return QGEMM_ERR_UNSUPPORTED;
+}
+
+int launch_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t N, hipStream_t stream) {
+    if (M == 0 || N == 0) return QGEMM_OK;
+    if (M >= ((size_t)1 << 31) || N >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
+    dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+    if (grid.y > 65535u * 1024u) return QGEMM_ERR_TOO_LARGE;
+    switch (elem_bytes) {
+        case 1:
+            hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, dim3(256), 0, stream, (const uint8_t *)in, (uint8_t *)out,
+                               (uint32_t)M, (uint32_t)N);
+            break;
+        case 2:
+            hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, stream, (const uint16_t *)in,
+                               (uint16_t *)out, (uint32_t)M, (uint32_t)N);
+            break;
+        case 4:
+            hipLaunchKernelGGL(transpose_kernel<uint32_t>, grid, dim3(256), 0, stream, (const uint32_t *)in,
+                               (uint32_t *)out, (uint32_t)M, (uint32_t)N);
+            break;
+        default: return QGEMM_ERR_UNSUPPORTED;
+    }
+    return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
+}
+
+}  // namespace
+
+// ===========================================================================
+extern "C" {
+
+QGEMM_EXPORT int qgemm_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+QGEMM_EXPORT int qgemm_init(void) {
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    return ensure_init_locked();
+}
+
+QGEMM_EXPORT int qgemm_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (g_ctx.workspace) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(g_ctx.workspace);
+    }
+    g_ctx.workspace = nullptr;
+    g_ctx.workspace_bytes = 0;
+    g_ctx.ready = false;
+    return QGEMM_OK;
+}
+
+QGEMM_EXPORT const char *qgemm_status_string(int status) {
+    switch (status) {
+        case QGEMM_OK: return "ok";
+        case QGEMM_ERR_INVALID_ARG: return "invalid argument";
+        case QGEMM_ERR_UNSUPPORTED: return "unsupported dtype / layout combination";
+        case QGEMM_ERR_NO_DEVICE: return "no HIP device";
+        case QGEMM_ERR_LAUNCH: return "HIP call failed";
+        case QGEMM_ERR_ALLOC: return "workspace allocation failed";
+        case QGEMM_ERR_NOT_DIVISIBLE_M: return "M is not divisible by any predefined BLOCK_TILE_SIZE_M in the list";
+        case QGEMM_ERR_NOT_DIVISIBLE_N: return "N is not divisible by any predefined BLOCK_TILE_SIZE_N in the list";
+        case QGEMM_ERR_NOT_DIVISIBLE_K: return "K is not divisible by any predefined BLOCK_TILE_SIZE_K in the list";
+        case QGEMM_ERR_TOO_LARGE: return "dimension or stride too large";
+    }
+    return "unknown status";
+}
+
+QGEMM_EXPORT int qgemm_tile_map(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n, uint32_t group_m, uint32_t *tile_m,
+                   uint32_t *tile_n) {
+    if (!tile_m || !tile_n || tiles_m == 0 || tiles_n == 0) return QGEMM_ERR_INVALID_ARG;
+    if ((uint64_t)wg >= (uint64_t)tiles_m * tiles_n) return QGEMM_ERR_INVALID_ARG;
+    tile_map(wg, tiles_m, tiles_n, group_m, *tile_m, *tile_n);
+    return QGEMM_OK;
+}
+
+QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
+    if (!key) return QGEMM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (!std::strcmp(key, "force_config")) g_ctx.force_config = value;
+    else if (!std::strcmp(key, "force_split")) g_ctx.force_split = value;
+    else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
+    else return QGEMM_ERR_INVALID_ARG;
+    return QGEMM_OK;
+}
+
+QGEMM_EXPORT int qgemm_last_config(char *buf, size_t buflen) {
+    if (!buf || buflen == 0) return QGEMM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    std::snprintf(buf, buflen, "%s", g_ctx.last_config.c_str());
+    return QGEMM_OK;
+}
+
+QGEMM_EXPORT int qgemm_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t N, void *stream) {
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) return QGEMM_ERR_UNSUPPORTED;
+    if (M == 0 || N == 0) return QGEMM_OK;
+    if (!in || !out) return QGEMM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    int st = ensure_init_locked();
+    if (st != QGEMM_OK) return st;
+    return launch_transpose(elem_bytes, in, out, M, N, (hipStream_t)stream);
+}
+
+QGEMM_EXPORT int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const void *A, size_t ldA, const void *B, size_t ldB,
+               void *C, size_t ldC, size_t M, size_t N, size_t K, void *stream_) {
+    const int arith = arith_of(in_dtype);
+    if (arith < 0 || !out_dtype_ok(in_dtype, out_dtype)) return QGEMM_ERR_UNSUPPORTED;
+    if (layout_b != QGEMM_B_KN && layout_b != QGEMM_B_NK) return QGEMM_ERR_INVALID_ARG;
+    if (M == 0 || N == 0) return QGEMM_OK;
+    if (!A || !B || !C || K == 0) return QGEMM_ERR_INVALID_ARG;
+    if (ldA < K || ldC < N || ldB < (layout_b == QGEMM_B_KN ? N : K)) return QGEMM_ERR_INVALID_ARG;
+    hipStream_t stream = (hipStream_t)stream_;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    int st = ensure_init_locked();
+    if (st != QGEMM_OK) return st;
+
+    const size_t eb = dtype_bytes(in_dtype);
+    NtProblem q;
+    std::memset(&q, 0, sizeof(q));
+    q.arith = arith;
+    q.block = false;
+    q.A = A;
+    q.C = C;
+    q.lda_bytes = ldA * eb;
+    q.ldc = ldC;
+    q.M = M;
+    q.N = N;
+    q.Kbytes = K * eb;
+    q.out_dtype = out_dtype;
+    q.per_matrix = 0;
+    q.split_k = 0;
+
+    if (layout_b == QGEMM_B_NK) {
+        q.B = B;
+        q.ldb_bytes = ldB * eb;
+        if (mfma_shape_ok(q) && aligned16(A) && aligned16(B)) return launch_nt(q, stream);
+    } else if (ldB == N) {
+        // "NN": bring B to N x K through the transpose utility (the route the reference's
+        // v3.1 launcher sketches, sm80_gemm_kernel_v3.1.cu:277-279), then run the NT kernel.
+        q.ldb_bytes = K * eb;
+        if (mfma_shape_ok(q) && aligned16(A)) {
+            Plan pl;
+            st = plan_nt(q, pl);
+            if (st != QGEMM_OK) return st;
+            const size_t split_room = (pl.split_bytes + 255) / 256 * 256;
+            void *ws = nullptr;
+            st = ensure_workspace_locked(split_room + N * K * eb, &ws);
+            if (st != QGEMM_OK) return st;
+            void *bt = (char *)ws + split_room;
+            st = launch_transpose((int)eb, B, bt, K, N, stream);
+            if (st != QGEMM_OK) return st;
+            q.B = bt;
+            return run_nt(q, pl, ws, stream);
+        }
+    }
+
+    StridedArgs s;
+    std::memset(&s, 0, sizeof(s));
+    s.A = A;
+    s.B = B;
+    s.C = C;
+    s.M = (uint32_t)M;
+    s.N = (uint32_t)N;
+    s.K = (uint32_t)K;
+    s.a_rs = ldA;
+    s.a_cs = 1;
+    if (layout_b == QGEMM_B_NK) {
+        s.b_ns = ldB;
+        s.b_ks = 1;
+    } else {
+        s.b_ns = 1;
+        s.b_ks = ldB;
+    }
+    s.ldc = ldC;
+    s.out_dtype = out_dtype;
+    s.scale_mode = 0;
+    return launch_strided(in_dtype, s, stream);
+}
+
+QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
+                      const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N, size_t K,
+                      int split_k, void *stream_) {
+    if (in_dtype != QGEMM_DT_I8 && in_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
+    if (!out_dtype_ok(in_dtype, out_dtype)) return QGEMM_ERR_UNSUPPORTED;
+    if (scale_mode != QGEMM_SCALE_PER_MATRIX && scale_mode != QGEMM_SCALE_BLOCK128) return QGEMM_ERR_INVALID_ARG;
+    if (scale_mode == QGEMM_SCALE_BLOCK128 && in_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
+    if (layout != QGEMM_LAYOUT_K_CONTIGUOUS && layout != QGEMM_LAYOUT_REFERENCE) return QGEMM_ERR_INVALID_ARG;
+    if (split_k < 0) return QGEMM_ERR_INVALID_ARG;
+    if (layout == QGEMM_LAYOUT_REFERENCE) {
+        // dispatch contract of select_BLOCK_TILE_SIZE_{M,N,K}: hip_mix_gemm_kernel.cpp:442-505
+        if (M % 32 != 0) return QGEMM_ERR_NOT_DIVISIBLE_M;
+        if (N % 32 != 0) return QGEMM_ERR_NOT_DIVISIBLE_N;
+        if (K % 32 != 0) return QGEMM_ERR_NOT_DIVISIBLE_K;
+    }
+    if (M == 0 || N == 0) return QGEMM_OK;
+    if (!A || !B || !C || K == 0 || ldC < N) return QGEMM_ERR_INVALID_ARG;
+    const bool raw_acc = out_dtype == QGEMM_DT_I32;
+    if (!raw_acc && (!a_scale || !b_scale)) return QGEMM_ERR_INVALID_ARG;
+    hipStream_t stream = (hipStream_t)stream_;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    int st = ensure_init_locked();
+    if (st != QGEMM_OK) return st;
+
+    const bool block = scale_mode == QGEMM_SCALE_BLOCK128;
+    const uint32_t KB = (uint32_t)((K + 127) / 128), NBLK = (uint32_t)((N + 127) / 128);
+    NtProblem q;
+    std::memset(&q, 0, sizeof(q));
+    q.arith = arith_of(in_dtype);
+    q.block = block;
+    q.C = C;
+    q.ldc = ldC;
+    q.M = M;
+    q.N = N;
+    q.Kbytes = K;
+    q.lda_bytes = K;
+    q.ldb_bytes = K;
+    q.as = a_scale;
+    q.bs = b_scale;
+    q.out_dtype = out_dtype;
+    q.per_matrix = (!block && !raw_acc) ? 1 : 0;
+    q.split_k = split_k;
+    if (block) {
+        if (layout == QGEMM_LAYOUT_K_CONTIGUOUS) {
+            q.as_ms = KB; q.as_ks = 1; q.bs_ns = KB; q.bs_ks = 1;
+        } else {   // a_scale[m + kb*M], b_scale[nb + kb*ceil(N/128)]: hip_mix_gemm_kernel.cpp:137,149,164
+            q.as_ms = 1; q.as_ks = (uint32_t)M; q.bs_ns = 1; q.bs_ks = NBLK;
+        }
+    }
+
+    if (layout == QGEMM_LAYOUT_K_CONTIGUOUS) {
+        q.A = A;
+        q.B = B;
+        if (mfma_shape_ok(q) && aligned16(A) && aligned16(B)) return launch_nt(q, stream);
+    } else if (mfma_shape_ok(q)) {
+        // reference layout: A is K x M (M contiguous), B is K x N.  Bring both to K-contiguous
+        // through the transpose utility, then run the NT kernel.
+        Plan pl;
+        st = plan_nt(q, pl);
+        if (st != QGEMM_OK) return st;
+        const size_t split_room = (pl.split_bytes + 255) / 256 * 256;
+        const size_t at_bytes = (M * K + 255) / 256 * 256;
+        void *ws = nullptr;
+        st = ensure_workspace_locked(split_room + at_bytes + N * K, &ws);
+        if (st != QGEMM_OK) return st;
+        char *at = (char *)ws + split_room, *bt = at + at_bytes;
+        st = launch_transpose(1, A, at, K, M, stream);
+        if (st != QGEMM_OK) return st;
+        st = launch_transpose(1, B, bt, K, N, stream);
+        if (st != QGEMM_OK) return st;
+        q.A = at;
+        q.B = bt;
+        return run_nt(q, pl, ws, stream);
+    }
+
+    StridedArgs s;
+    std::memset(&s, 0, sizeof(s));
+    s.A = A;
+    s.B = B;
+    s.C = C;
+    s.as = a_scale;
+    s.bs = b_scale;
+    s.M = (uint32_t)M;
+    s.N = (uint32_t)N;
+    s.K = (uint32_t)K;
+    if (layout == QGEMM_LAYOUT_K_CONTIGUOUS) {
+        s.a_rs = K; s.a_cs = 1; s.b_ns = K; s.b_ks = 1;
+    } else {
+        s.a_rs = 1; s.a_cs = M; s.b_ns = 1; s.b_ks = N;
+    }
+    s.ldc = ldC;
+    s.as_ms = q.as_ms; s.as_ks = q.as_ks; s.bs_ns = q.bs_ns; s.bs_ks = q.bs_ks;
+    // partial products per reference K tile: first of {128, 64, 32} dividing K (:442-463)
+    s.bk = K % 128 == 0 ? 128 : (K % 64 == 0 ? 64 : (K % 32 == 0 ? 32 : 128));
+    s.out_dtype = out_dtype;
+    s.scale_mode = raw_acc ? 0 : scale_mode;
+    return launch_strided(in_dtype, s, stream);
+}
+
+// ---------------------------------------------------------------------------
+// self test
+// ---------------------------------------------------------------------------
+namespace {
+
+float host_decode(int arith, const uint8_t *p, int idx) {
+    if (arith == AR_I8) return (float)((const int8_t *)p)[idx];
+    if (arith == AR_F8) {
+        const uint8_t b = p[idx];
+        const int e = (b >> 3) & 15, m = b & 7;
+        float mag = e == 0 ? (float)m / 512.0f : (1.0f + (float)m / 8.0f) * std::exp2((float)(e - 7));
+        return (b & 0x80) ? -mag : mag;
+    }
+    uint16_t h;
+    std::memcpy(&h, p + 2 * idx, 2);
+    if (arith == AR_BF16) {
+        uint32_t u = (uint32_t)h << 16;
+        float f;
+        std::memcpy(&f, &u, 4);
+        return f;
+    }
+    // fp16: the probe only uses small integers, exactly representable
+    const int e = (h >> 10) & 31, m = h & 1023;
+    float mag = e == 0 ? (float)m / 16777216.0f : (1.0f + (float)m / 1024.0f) * std::exp2((float)(e - 15));
+    return (h & 0x8000) ? -mag : mag;
+}
+
+// value v in [-4, 4] encoded in the family's element type
+void host_encode_small(int arith, int v, uint8_t *p, int idx) {
+    if (arith == AR_I8) { ((int8_t *)p)[idx] = (int8_t)v; return; }
+    if (arith == AR_F8) {
+        static const uint8_t code[5] = {0x00, 0x38, 0x40, 0x44, 0x48};   // 0, 1, 2, 3, 4
+        p[idx] = (uint8_t)(code[v < 0 ? -v : v] | (v < 0 ? 0x80 : 0));
+        return;
+    }
+    uint16_t h;
+    if (arith == AR_BF16) {
+        static const uint16_t code[5] = {0x0000, 0x3F80, 0x4000, 0x4040, 0x4080};
+        h = (uint16_t)(code[v < 0 ? -v : v] | (v < 0 ? 0x8000 : 0));
+    } else {
+        static const uint16_t code[5] = {0x0000, 0x3C00, 0x4000, 0x4200, 0x4400};
+        h = (uint16_t)(code[v < 0 ? -v : v] | (v < 0 ? 0x8000 : 0));
+    }
+    std::memcpy(p + 2 * idx, &h, 2);
+}
+
+}  // namespace
+
+QGEMM_EXPORT int qgemm_selftest_layouts(char *buf, size_t buflen) {
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    int st = ensure_init_locked();
+    if (st != QGEMM_OK) return st;
+    std::string rep;
+    bool all_ok = true;
+    char line[256];
+
+    // ---- LDS DMA: lane l's 16 bytes land at lds_base + 16*l, for low and high LDS addresses;
+    //      out-of-range lanes write zeros
+    {
+        const int nsrc = 4096;
+        std::vector<uint8_t> hsrc(nsrc);
+        for (int i = 0; i < nsrc; ++i) hsrc[i] = (uint8_t)((i * 7 + (i >> 8)) & 0xFF);
+        std::vector<uint32_t> hoff(64);
+        for (int l = 0; l < 64; ++l) hoff[l] = (uint32_t)(((63 - l) * 48) % 2048);   // a permutation-ish gather, 16-aligned
+        hoff[5] = 4096 + 64;   // out of range
+        hoff[40] = 0xFFFFFF00u;
+        void *dsrc = nullptr, *doff = nullptr, *dout = nullptr;
+        HIP_TRY(hipMalloc(&dsrc, nsrc));
+        HIP_TRY(hipMalloc(&doff, 256));
+        HIP_TRY(hipMalloc(&dout, 1024));
+        HIP_TRY(hipMemcpy(dsrc, hsrc.data(), nsrc, hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(doff, hoff.data(), 256, hipMemcpyHostToDevice));
+        HIP_TRY(hipFuncSetAttribute((const void *)probe_lds_dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    160 * 1024));
+        const uint32_t bases[3] = {0, 72 * 1024, 159 * 1024};
+        const uint32_t soffs[3] = {0, 1024, 16};
+        for (int t = 0; t < 3; ++t) {
+            hipLaunchKernelGGL(probe_lds_dma_kernel, dim3(1), dim3(64), 160 * 1024, 0, (const char *)dsrc,
+                               (const uint32_t *)doff, (uint32_t)nsrc, bases[t], soffs[t], (char *)dout);
+            HIP_TRY(hipGetLastError());
+            std::vector<uint8_t> hout(1024);
+            HIP_TRY(hipMemcpy(hout.data(), dout, 1024, hipMemcpyDeviceToHost));
+            int bad = 0, oob_zero = 0, oob_untouched = 0;
+            for (int l = 0; l < 64; ++l) {
+                const uint64_t off = (uint64_t)hoff[l] + soffs[t];
+                if (off + 16 > (uint64_t)nsrc) {
+                    bool z = true, u = true;
+                    for (int j = 0; j < 16; ++j) {
+                        z &= hout[l * 16 + j] == 0;
+                        u &= hout[l * 16 + j] == 0xA5;
+                    }
+                    oob_zero += z;
+                    oob_untouched += u;
+                    continue;
+                }
+                for (int j = 0; j < 16; ++j) bad += hout[l * 16 + j] != hsrc[off + j];
+            }
+            std::snprintf(line, sizeof(line), "lds_dma base=%u soffset=%u: mismatched_bytes=%d oob_lanes_zero=%d oob_lanes_untouched=%d\n",
+                          bases[t], soffs[t], bad, oob_zero, oob_untouched);
+            rep += line;
+            if (bad) all_ok = false;
+        }
+        (void)hipFree(dsrc);
+        (void)hipFree(doff);
+        (void)hipFree(dout);
+    }
+
+    // ---- MFMA operand / accumulator layout for the four families
+    {
+        void *dx = nullptr, *dy = nullptr, *dout = nullptr;
+        HIP_TRY(hipMalloc(&dx, 2048));
+        HIP_TRY(hipMalloc(&dy, 2048));
+        HIP_TRY(hipMalloc(&dout, 1024));
+        const char *names[4] = {"i8", "f8", "bf16", "f16"};
+        for (int arith = 0; arith < 4; ++arith) {
+            const int eb = arith <= AR_F8 ? 1 : 2;
+            const int per_lane = 32 / eb;                    // elements per lane per operand
+            std::vector<uint8_t> hx(2048), hy(2048);
+            uint32_t rng = 12345u + arith;
+            auto next = [&]() { rng = rng * 1664525u + 1013904223u; return (int)((rng >> 24) % 9) - 4; };
+            for (int i = 0; i < 64 * per_lane; ++i) {
+                host_encode_small(arith, next(), hx.data(), i);
+                host_encode_small(arith, next(), hy.data(), i);
+            }
+            HIP_TRY(hipMemcpy(dx, hx.data(), 2048, hipMemcpyHostToDevice));
+            HIP_TRY(hipMemcpy(dy, hy.data(), 2048, hipMemcpyHostToDevice));
+            switch (arith) {
+                case AR_I8: hipLaunchKernelGGL(probe_mfma_kernel<AR_I8>, dim3(1), dim3(64), 0, 0, (const char *)dx, (const char *)dy, (int *)dout); break;
+                case AR_F8: hipLaunchKernelGGL(probe_mfma_kernel<AR_F8>, dim3(1), dim3(64), 0, 0, (const char *)dx, (const char *)dy, (int *)dout); break;
+                case AR_BF16: hipLaunchKernelGGL(probe_mfma_kernel<AR_BF16>, dim3(1), dim3(64), 0, 0, (const char *)dx, (const char *)dy, (int *)dout); break;
+                default: hipLaunchKernelGGL(probe_mfma_kernel<AR_F16>, dim3(1), dim3(64), 0, 0, (const char *)dx, (const char *)dy, (int *)dout); break;
+            }
+            HIP_TRY(hipGetLastError());
+            std::vector<int> hout(256);
+            HIP_TRY(hipMemcpy(hout.data(), dout, 1024, hipMemcpyDeviceToHost));
+            // assumed: operand lane l = row (l & 15), K group (l >> 4); the same element position of
+            // the two operands meets in the contraction; accumulator lane l, register r =
+            // D[first-operand row 4*(l >> 4) + r][second-operand row (l & 15)]
+            int bad = 0;
+            for (int l = 0; l < 64; ++l)
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 4 * (l >> 4) + r, j = l & 15;
+                    double sum = 0;
+                    for (int g = 0; g < 4; ++g)
+                        for (int e = 0; e < per_lane; ++e)
+                            sum += (double)host_decode(arith, hx.data(), (g * 16 + i) * per_lane + e) *
+                                   (double)host_decode(arith, hy.data(), (g * 16 + j) * per_lane + e);
+                    double got;
+                    if (arith == AR_I8) got = (double)hout[l * 4 + r];
+                    else {
+                        float f;
+                        std::memcpy(&f, &hout[l * 4 + r], 4);
+                        got = (double)f;
+                    }
+                    bad += got != sum;
+                }
+            std::snprintf(line, sizeof(line), "mfma %s: mismatched_accumulators=%d of 256\n", names[arith], bad);
+            rep += line;
+            if (bad) all_ok = false;
+        }
+        (void)hipFree(dx);
+        (void)hipFree(dy);
+        (void)hipFree(dout);
+    }
+    if (buf && buflen) std::snprintf(buf, buflen, "%s", rep.c_str());
+    return all_ok ? QGEMM_OK : QGEMM_ERR_UNSUPPORTED;
+}
+
+}  // extern "C"

@@ -1,0 +1,46 @@
+// Probes of the hardware behaviour the GEMM kernels are built on.  The gfx950
+// counterpart of the reference's playground/ (ldmatrix / movmatrix lane-layout
+// probes): each probe runs one wave and the host compares what came back with
+// the layout the kernels assume.
+#pragma once
+#include "gemm_mfma.cuh"
+
+namespace qgemm {
+
+// One wave fetches 64 x 16 bytes from `src` with per-lane byte offsets `voff`
+// through buffer_load_dwordx4 ... lds into LDS at `lds_base`, then copies the
+// 1 KiB at lds_base back to `out`.  LDS is pre-filled with 0xA5 so "not written"
+// and "written with zeros" can be told apart.  `range` is the buffer size: lanes
+// whose offset lies beyond it are out of range.
+__global__ void __launch_bounds__(64) probe_lds_dma_kernel(const char *src, const uint32_t *voff, uint32_t range,
+                                                           uint32_t lds_base, uint32_t soffset, char *out) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    const int lane = threadIdx.x;
+    *(v4i *)(smem + lds_base + lane * 16) = v4i{(int)0xA5A5A5A5, (int)0xA5A5A5A5, (int)0xA5A5A5A5, (int)0xA5A5A5A5};
+    __syncthreads();
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(src, range);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void *)(smem + lds_base), 16, voff[lane], soffset, 0, 0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __syncthreads();
+    *(v4i *)(out + lane * 16) = *(const v4i *)(smem + lds_base + lane * 16);
+#endif
+}
+
+// One MFMA on operands taken verbatim from memory: lane l's first operand is the
+// 32 bytes at x + 32*l, second operand at y + 32*l (the 16-byte MFMAs use the
+// first 16 of each and then the second 16, exactly like mma128).  Accumulator
+// registers go to out[4*l .. 4*l+3] (raw 32-bit).
+template <int ARITH>
+__global__ void __launch_bounds__(64) probe_mfma_kernel(const char *x, const char *y, int *out) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int lane = threadIdx.x;
+    const v4i x0 = *(const v4i *)(x + lane * 32), x1 = *(const v4i *)(x + lane * 32 + 16);
+    const v4i y0 = *(const v4i *)(y + lane * 32), y1 = *(const v4i *)(y + lane * 32 + 16);
+    typename AccT<ARITH>::type c = {0, 0, 0, 0};
+    c = mma128<ARITH>(x0, x1, y0, y1, c);
+    for (int r = 0; r < 4; ++r) out[lane * 4 + r] = __builtin_bit_cast(int, c[r]);
+#endif
+}
+
+}  // namespace qgemm

@@ -1,0 +1,25 @@
+// Table of compiled MFMA GEMM variants (one row per tile shape, loader and
+// arithmetic family).  Plays the role of the reference's constexpr tile tables
+// (src/include/gemm_config.h:30-36,65-71) and of its divisibility dispatch
+// (hip_mix_gemm_kernel.cpp:442-505), but is chosen at run time from the shape.
+#pragma once
+#include "gemm_mfma.cuh"
+
+namespace qgemm {
+
+struct Variant {
+    const char *name;
+    int arith;
+    bool block_scale;
+    int bm, bn, threads, lds_bytes, loader;
+    hipError_t (*launch)(const GemmArgs &, uint32_t grid, hipStream_t);
+};
+
+// one translation unit per arithmetic family defines one of these
+const Variant *variants_i8(int *count);
+const Variant *variants_f8(int *count);
+const Variant *variants_f8_block(int *count);
+const Variant *variants_bf16(int *count);
+const Variant *variants_f16(int *count);
+
+}  // namespace qgemm

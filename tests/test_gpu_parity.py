@@ -1,0 +1,309 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU
+oracle on the same seeded inputs.  Integer results bit-exact; float results
+within rtol 2e-2 / atol 1e-2 of the fp32-accumulate oracle (tests/util.py).
+
+Sizes here are ones the oracle finishes in seconds; the full BASELINE sizes are
+in test_gpu_full_size.py."""
+import numpy as np
+import pytest
+import torch
+
+import qgemm_amd as Q
+from oracle import cpu_ref as R
+from tests.util import (assert_close, dev, fp8_inputs, fp8_tensor, host, int8_inputs, say, scalar)
+
+pytestmark = pytest.mark.gpu
+
+N_VARIANTS = 9          # rows of the variant table in qgemm_amd/csrc/gemm_inst.hip
+
+
+@pytest.fixture(autouse=True)
+def _reset_options():
+    yield
+    Q.set_option("force_config", -1)
+    Q.set_option("force_split", 0)
+    Q.set_option("group_m", 0)
+
+
+def test_selftest_layouts():
+    """The hardware behaviour the kernels assume: LDS-DMA placement (also above 64 KiB),
+    MFMA operand and accumulator lane layouts for i8 / f8 / bf16 / f16."""
+    say("selftest_layouts")
+    ok, report = Q.selftest_layouts()
+    print(report, flush=True)
+    assert ok, report
+
+
+# ----------------------------------------------------------------- int8
+@pytest.mark.parametrize("variant", range(N_VARIANTS))
+@pytest.mark.parametrize("shape", [(256, 256, 256), (300, 202, 384), (16, 128, 128), (520, 1000, 640)])
+def test_int8_accumulators_bit_exact_every_variant(variant, shape):
+    M, N, K = shape
+    say("int8 i32", shape, "variant", variant)
+    qa, sa, qb, sb = int8_inputs(M, N, K, seed=100 + variant)
+    ref = R.gemm_i8_i32(qa, qb)
+    Q.set_option("force_config", variant)
+    c = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+    Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), c, split_k=1)
+    assert np.array_equal(host(c), ref), Q.last_config()
+
+
+@pytest.mark.parametrize("shape", [(512, 384, 1024), (100, 36, 256)])
+def test_int8_per_matrix_f32_bit_exact(shape):
+    M, N, K = shape
+    say("int8 f32", shape)
+    qa, sa, qb, sb = int8_inputs(M, N, K, seed=7)
+    ref = R.scale_i32_to_f32(R.gemm_i8_i32(qa, qb), sa, sb)
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), c)
+    assert np.array_equal(host(c), ref), Q.last_config()      # one rounding each side: identical bits
+
+
+def test_int8_extremes_do_not_overflow():
+    M, N, K = 32, 128, 8192
+    say("int8 extremes", (M, N, K))
+    a = torch.full((M, K), 127, dtype=torch.int8, device="cuda")
+    b = torch.full((N, K), -127, dtype=torch.int8, device="cuda")
+    c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    Q.int8_mm(a, b, scalar(1), scalar(1), c)
+    assert torch.all(c == -127 * 127 * K)
+
+
+@pytest.mark.parametrize("nsplit", [2, 3, 8])
+def test_int8_split_k_bit_exact(nsplit):
+    M, N, K = 64, 384, 2048
+    say("int8 split-k", nsplit)
+    qa, sa, qb, sb = int8_inputs(M, N, K, seed=11)
+    acc = R.gemm_i8_i32(qa, qb)
+    c32 = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), c32, split_k=nsplit)
+    assert "splitk" in Q.last_config()
+    assert np.array_equal(host(c32), acc)
+    cf = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), cf, split_k=nsplit)
+    assert np.array_equal(host(cf), R.scale_i32_to_f32(acc, sa, sb))
+
+
+# ------------------------------------------------------------------ fp8
+@pytest.mark.parametrize("variant", range(N_VARIANTS))
+def test_fp8_per_matrix_every_variant(variant):
+    M, N, K = 272, 392, 512
+    say("fp8 per-matrix", (M, N, K), "variant", variant)
+    qa, sa, qb, sb = fp8_inputs(M, N, K, seed=200 + variant)
+    ref = R.gemm_f32acc(R.decode_fp8(qa), R.decode_fp8(qb)) * np.float32(sa * sb)
+    Q.set_option("force_config", variant)
+    for dt in (torch.bfloat16, torch.float32, torch.float16):
+        c = torch.zeros((M, N), dtype=dt, device="cuda")
+        Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), scalar(sa), scalar(sb), c, M, N, K, Q.SCALE_PER_MATRIX,
+                      split_k=1)
+        assert_close(host(c).astype(np.float32), ref, what=f"{Q.last_config()} {dt}")
+
+
+def test_fp8_exact_on_small_integers():
+    """Products of small integers sum exactly in fp32: the GPU result must equal the oracle bit for bit,
+    which pins operand order and the K mapping without any tolerance."""
+    M, N, K = 128, 256, 1024
+    say("fp8 exact integers")
+    rng = np.random.default_rng(5)
+    a = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    b = rng.integers(-4, 5, size=(N, K)).astype(np.float32)
+    qa, qb = R.encode_fp8(a), R.encode_fp8(b)
+    ref = R.gemm_f32acc(a, b)
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), scalar(1), scalar(1), c, M, N, K, Q.SCALE_PER_MATRIX)
+    assert np.array_equal(host(c), ref)
+
+
+def test_fp8_every_code_decodes_like_the_oracle():
+    """Row i of A holds code i on the diagonal position i: C = A * I picks every finite e4m3 code once."""
+    say("fp8 all codes")
+    codes = np.array([b for b in range(256) if (b & 0x7F) != 0x7F], np.uint8)
+    M, K, N = 256, 256, 256
+    qa = np.zeros((M, K), np.uint8)
+    for i, cde in enumerate(codes):
+        qa[i, i] = cde
+    qb = np.zeros((N, K), np.uint8)
+    qb[np.arange(N), np.arange(N)] = 0x38          # 1.0
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), scalar(1), scalar(1), c, M, N, K, Q.SCALE_PER_MATRIX)
+    got = host(c)
+    assert np.array_equal(np.diag(got)[: len(codes)], R.decode_fp8(codes))
+
+
+@pytest.mark.parametrize("variant", range(N_VARIANTS))
+def test_fp8_block_scaled_every_variant(variant):
+    M, N, K = 160, 384, 512
+    say("fp8 block-scaled", (M, N, K), "variant", variant)
+    qa, _, qb, _ = fp8_inputs(M, N, K, seed=300 + variant)
+    as_ = R.fill_uniform((M, K // 128), 301, 0.5, 2.0)
+    bs = R.fill_uniform((N // 128, K // 128), 302, 0.5, 2.0)
+    # bring the products to O(1) so atol means something
+    as_ *= np.float32(1.0 / 448.0)
+    bs *= np.float32(1.0 / 448.0)
+    ref = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)
+    Q.set_option("force_config", variant)
+    c = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128, split_k=1)
+    assert_close(host(c), ref, what=Q.last_config())
+
+
+def test_fp8_block_scaled_power_of_two_scales_bit_exact():
+    """Power-of-two scales commute exactly with fp32 arithmetic, and small-integer products sum exactly:
+    the scaled result must equal the oracle bit for bit (catches a wrong scale index)."""
+    M, N, K = 64, 256, 512
+    say("fp8 block pow2")
+    rng = np.random.default_rng(6)
+    a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+    as_ = (2.0 ** rng.integers(-3, 4, size=(M, K // 128))).astype(np.float32)
+    bs = (2.0 ** rng.integers(-3, 4, size=(N // 128, K // 128))).astype(np.float32)
+    ref = R.gemm_fp8_block(a, b, as_, bs)
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K,
+                  Q.SCALE_BLOCK128)
+    assert np.array_equal(host(c), ref)
+
+
+def test_fp8_mm_reference_layout():
+    """fp8_mm(a, b, as, bs, c) with the reference's column-major contract
+    (hip_mix_gemm_kernel.cpp:425-439): same numbers as the K-contiguous call."""
+    M, N, K = 128, 192, 384
+    say("fp8_mm reference layout")
+    qa, _, qb, _ = fp8_inputs(M, N, K, seed=31)
+    as_ = R.fill_uniform((M, K // 128), 32, 0.5, 2.0) / np.float32(448)
+    bs = R.fill_uniform(((N + 127) // 128, K // 128), 33, 0.5, 2.0) / np.float32(448)
+    ref = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)
+    # column-major [m,k] == row-major [k,m]; torch views with the reference's sizes and strides
+    a_t = fp8_tensor(np.ascontiguousarray(qa.T)).t()          # size (M,K), stride (1,M)
+    b_t = fp8_tensor(np.ascontiguousarray(qb.T)).t()          # size (N,K), stride (1,N)
+    as_t = dev(np.ascontiguousarray(as_.T)).t()
+    bs_t = dev(np.ascontiguousarray(bs.T)).t()
+    c = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.fp8_mm(a_t, b_t, as_t, bs_t, c)
+    assert_close(host(c), ref, what=Q.last_config())
+    # the oracle in the reference's own layout gives the same numbers
+    tn = R.gemm_fp8_block(R.decode_fp8(np.ascontiguousarray(qa.T)), R.decode_fp8(np.ascontiguousarray(qb.T)),
+                          np.ascontiguousarray(as_.T), np.ascontiguousarray(bs.T), "tn", "col")
+    assert np.array_equal(tn, ref)
+
+
+def test_fp8_mm_dispatch_errors_like_the_reference():
+    """hip_mix_gemm_kernel.cpp:460,485,503: dimensions not divisible by 32 throw."""
+    say("fp8_mm errors")
+    z = torch.zeros(1, device="cuda")
+    for (m, n, k), status in (((48, 64, 128), 6), ((64, 48, 128), 7), ((64, 64, 80), 8)):
+        a = torch.zeros((k, m), dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn).t()
+        b = torch.zeros((k, n), dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn).t()
+        c = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+        with pytest.raises(Q.QgemmError) as e:
+            Q.fp8_mm(a, b, z, z, c)
+        assert e.value.status == status and "not divisible" in str(e.value)
+
+
+@pytest.mark.parametrize("shape", [(64, 64, 96), (32, 96, 160), (33, 17, 50)])
+def test_any_shape_kernel_k_not_multiple_of_128(shape):
+    M, N, K = shape
+    say("any-shape", shape)
+    qa, sa, qb, sb = int8_inputs(M, N, K, seed=41)
+    c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), c)
+    assert Q.last_config() == "strided_any_shape"
+    assert np.array_equal(host(c), R.gemm_i8_i32(qa, qb))
+    qa, sa, qb, sb = fp8_inputs(M, N, K, seed=42)
+    if K % 32 == 0 and M % 32 == 0 and N % 32 == 0:
+        as_ = R.fill_uniform((M, (K + 127) // 128), 43, 0.5, 2.0) / np.float32(448)
+        bs = R.fill_uniform(((N + 127) // 128, (K + 127) // 128), 44, 0.5, 2.0) / np.float32(448)
+        ref = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)      # bk by the reference's dispatch
+        cb = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), dev(as_), dev(bs), cb, M, N, K, Q.SCALE_BLOCK128)
+        assert_close(host(cb), ref)
+    ref = R.gemm_f32acc(R.decode_fp8(qa), R.decode_fp8(qb)) * np.float32(sa * sb)
+    cf = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), scalar(sa), scalar(sb), cf, M, N, K, Q.SCALE_PER_MATRIX)
+    assert_close(host(cf), ref)
+
+
+@pytest.mark.parametrize("nsplit", [2, 4])
+def test_fp8_split_k(nsplit):
+    M, N, K = 16, 512, 2048
+    say("fp8 split-k", nsplit)
+    qa, sa, qb, sb = fp8_inputs(M, N, K, seed=51)
+    ref = R.gemm_f32acc(R.decode_fp8(qa), R.decode_fp8(qb)) * np.float32(sa * sb)
+    c = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), scalar(sa), scalar(sb), c, M, N, K, Q.SCALE_PER_MATRIX,
+                  split_k=nsplit)
+    assert "splitk" in Q.last_config()
+    assert_close(host(c), ref)
+    # block-scaled + split: partial planes are already scaled
+    as_ = R.fill_uniform((M, K // 128), 52, 0.5, 2.0) / np.float32(448)
+    bs = R.fill_uniform((N // 128, K // 128), 53, 0.5, 2.0) / np.float32(448)
+    refb = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128, split_k=nsplit)
+    assert_close(host(c), refb)
+
+
+# ---------------------------------------------------------- plain fp16 / bf16
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("layout_b", ["nk", "kn"])
+@pytest.mark.parametrize("shape", [(256, 256, 256), (136, 200, 192)])
+def test_plain_gemm_16bit(dtype, layout_b, shape):
+    M, N, K = shape
+    say("plain", dtype, layout_b, shape)
+    enc, dec, tdt = ((R.encode_f16, R.decode_f16, torch.float16) if dtype == "f16"
+                     else (R.encode_bf16, R.decode_bf16, torch.bfloat16))
+    ha, hb = enc(R.fill_uniform((M, K), 61)), enc(R.fill_uniform((N, K), 62))     # cfg 1: uniform[-1, 1]
+    ref = R.gemm_f32acc(dec(ha), dec(hb))
+    a = dev(ha.view(np.int16)).view(tdt)
+    b_nk = dev(hb.view(np.int16)).view(tdt)
+    b = b_nk if layout_b == "nk" else b_nk.t().contiguous()
+    for out_dt in (tdt, torch.float32):
+        c = torch.zeros((M, N), dtype=out_dt, device="cuda")
+        Q.gemm(a, b, c, layout_b)
+        got = host(c).astype(np.float32) if out_dt != torch.bfloat16 else host(c)
+        # 16-bit output: half an ulp of the output type on top of the accumulation-order slack
+        rtol = 2.0 ** -8 if out_dt == torch.bfloat16 else (2.0 ** -10 if out_dt == torch.float16 else 1e-5)
+        assert_close(got, ref, rtol=rtol, atol=1e-3, what=f"{Q.last_config()} {out_dt}")
+
+
+def test_plain_gemm_reference_pattern_inputs():
+    """The harness's closed-form inputs and check (tests/includes/test_config.h:251-258, 161-169):
+    bf16 in, fp32 out, NN layout, max |C - ref| < 5e-2."""
+    M = N = K = 256
+    say("pattern inputs", (M, N, K))
+    ha = R.encode_bf16(R.fill_pattern((M, K), 0))
+    hb = R.encode_bf16(R.fill_pattern((K, N), 1))
+    ref = R.gemm_f32acc(R.decode_bf16(ha), R.decode_bf16(hb), "nn")
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.gemm(dev(ha.view(np.int16)).view(torch.bfloat16), dev(hb.view(np.int16)).view(torch.bfloat16), c, "kn")
+    assert R.max_abs_diff(host(c), ref) < 5e-2
+
+
+# ------------------------------------------------------------------ transpose
+@pytest.mark.parametrize("dt", [torch.uint8, torch.int16, torch.float32])
+@pytest.mark.parametrize("shape", [(64, 32), (128, 256), (100, 36), (1, 77), (1024, 1024)])
+def test_transpose(dt, shape):
+    M, N = shape
+    say("transpose", dt, shape)
+    a = np.random.default_rng(1).integers(0, 120, size=(M, N))
+    x = torch.from_numpy(a).to(dt).cuda()
+    y = torch.zeros((N, M), dtype=dt, device="cuda")
+    Q.matrix_transpose(x, y)
+    assert torch.equal(y, x.t().contiguous())
+    assert np.array_equal(host(y), R.transpose(host(x)))
+    back = torch.zeros_like(x)
+    Q.matrix_transpose(y, back)
+    assert torch.equal(back, x)                      # involution
+
+
+def test_empty_and_invalid_arguments():
+    say("empty / invalid")
+    z = torch.zeros((0, 16), dtype=torch.int8, device="cuda")
+    b = torch.zeros((16, 16), dtype=torch.int8, device="cuda")
+    c = torch.zeros((0, 16), dtype=torch.int32, device="cuda")
+    Q.int8_mm(z, b, scalar(1), scalar(1), c)          # M == 0: nothing to do, no error
+    with pytest.raises(Q.QgemmError) as e:            # int32 output is only defined for int8 input
+        Q.scaled_gemm(b.view(torch.float8_e4m3fn), b.view(torch.float8_e4m3fn), scalar(1), scalar(1),
+                      torch.zeros((16, 16), dtype=torch.int32, device="cuda"), 16, 16, 16, Q.SCALE_PER_MATRIX)
+    assert e.value.status == 2
+    with pytest.raises(ValueError):
+        Q.int8_mm(torch.zeros((16, 16), dtype=torch.int8), b, scalar(1), scalar(1), c)   # host tensor
