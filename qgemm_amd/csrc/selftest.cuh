@@ -39,7 +39,8 @@ __global__ void __launch_bounds__(64) probe_mfma_kernel(const char *x, const cha
     const v4i y0 = *(const v4i *)(y + lane * 32), y1 = *(const v4i *)(y + lane * 32 + 16);
     typename AccT<ARITH>::type c = {0, 0, 0, 0};
     c = mma128<ARITH>(x0, x1, y0, y1, c);
-    for (int r = 0; r < 4; ++r) out[lane * 4 + r] = __builtin_bit_cast(int, c[r]);
+    // (bit_cast of the whole vector: bit_cast of a single vector element reads element 0)
+    *(v4i *)(out + lane * 4) = __builtin_bit_cast(v4i, c);
 #endif
 }
 
