@@ -23,21 +23,27 @@ static hipError_t launch_variant(const GemmArgs &a, uint32_t grid, hipStream_t s
     return hipGetLastError();
 }
 
-#define ROW(NAME, BM, BN, WM_, WN_, LD)                                                                           \
-    {NAME, INST_ARITH, (bool)INST_BLOCK, BM, BN, GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD>::THREADS, \
-     GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD>::LDS_BYTES, LD,                                   \
-     &launch_variant<GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD>>}
+#define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP>
+#define ROWP(NAME, BM, BN, WM_, WN_, LD, PP, AUTO)                                                    \
+    {NAME, INST_ARITH, (bool)INST_BLOCK, BM, BN, CFG(BM, BN, WM_, WN_, LD, PP)::THREADS,             \
+     CFG(BM, BN, WM_, WN_, LD, PP)::LDS_BYTES, LD, AUTO, &launch_variant<CFG(BM, BN, WM_, WN_, LD, PP)>}
+#define ROW(NAME, BM, BN, WM_, WN_, LD, AUTO) ROWP(NAME, BM, BN, WM_, WN_, LD, PIPE_SIMPLE, AUTO)
 
+// Order matters: the heuristic walks the auto rows from large to small tiles, and
+// force_config indexes this table.  Block-scaled builds keep the simple pipeline for the
+// 256x256 tile (the in-loop rescale does not fit the ping-pong register budget).
 static const Variant kTable[] = {
-    ROW("256x256_w2x4_dma", 256, 256, 2, 4, LOAD_DMA),
-    ROW("256x128_w2x2_dma", 256, 128, 2, 2, LOAD_DMA),
-    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA),
-    ROW("64x128_w1x4_dma", 64, 128, 1, 4, LOAD_DMA),
-    ROW("32x128_w1x4_dma", 32, 128, 1, 4, LOAD_DMA),
-    ROW("16x128_w1x2_dma", 16, 128, 1, 2, LOAD_DMA),
-    ROW("256x256_w2x4_vgpr", 256, 256, 2, 4, LOAD_VGPR),
-    ROW("128x128_w2x2_vgpr", 128, 128, 2, 2, LOAD_VGPR),
-    ROW("32x128_w1x4_vgpr", 32, 128, 1, 4, LOAD_VGPR),
+    ROW("256x256_w2x4_dma", 256, 256, 2, 4, LOAD_DMA, false),
+    ROW("256x128_w2x2_dma", 256, 128, 2, 2, LOAD_DMA, false),
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, true),
+    ROW("64x128_w1x4_dma", 64, 128, 1, 4, LOAD_DMA, true),
+    ROW("32x128_w1x4_dma", 32, 128, 1, 4, LOAD_DMA, true),
+    ROW("16x128_w1x2_dma", 16, 128, 1, 2, LOAD_DMA, true),
+    ROW("256x256_w2x4_vgpr", 256, 256, 2, 4, LOAD_VGPR, (bool)INST_BLOCK),
+    ROW("128x128_w2x2_vgpr", 128, 128, 2, 2, LOAD_VGPR, false),
+    ROW("32x128_w1x4_vgpr", 32, 128, 1, 4, LOAD_VGPR, false),
+    ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, !(bool)INST_BLOCK),
+    ROWP("256x256_w2x4_pingpong", 256, 256, 2, 4, LOAD_DMA, PIPE_PINGPONG, false),
 };
 
 const Variant *INST_FN(int *count) {

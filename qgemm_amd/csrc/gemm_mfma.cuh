@@ -8,20 +8,26 @@
 // path are built around the CDNA4 matrix core.
 //
 // Data movement
-//   * A K step is 128 bytes of every tile row (128 fp8/int8 or 64 bf16/fp16).
-//   * Global -> LDS goes through buffer_load_dwordx4 ... lds (no VGPR staging).
-//     One such instruction moves a 1 KiB "fragment block": 16 tile rows x 64
-//     bytes of K.  Lane l fetches row (l & 15), bytes 16*(l >> 4) .. +16 of the
-//     64, and the hardware stores lane l's 16 bytes at block + 16*l.
-//   * That is exactly the operand order of the 16-row MFMA instructions (row =
-//     lane & 15, K group = lane >> 4), so a fragment is read back with one
-//     ds_read_b128 per lane at block + 16*lane: consecutive lanes read
-//     consecutive 16-byte words, which is free of bank conflicts by
-//     construction and needs no per-read address arithmetic.  (Which K bytes a
-//     lane group holds does not matter as long as A and B agree: the
-//     contraction index is summed away.)
-//   * LDS holds two stages (double buffer).  Tile k+1 is in flight while the
-//     matrix cores work on tile k; one s_barrier per K step.
+//   * A K step is 128 bytes of every tile row (128 fp8/int8 or 64 bf16/fp16):
+//     one full 128-byte cache line per row.
+//   * Global -> LDS goes through buffer_load_dwordx4 ... lds (no VGPR staging, no
+//     ds_write).  One such instruction moves 8 rows x 128 bytes = 1 KiB; lanes
+//     8r .. 8r+7 fetch the eight 16-byte chunks of row r, so every quad of lanes
+//     is one contiguous 64-byte request (the texture addresser only merges
+//     neighbouring lanes; one lane per row costs 4x the cycles).  The hardware
+//     stores lane l's 16 bytes at destination + 16*l.
+//   * LDS layout ("row block" = 16 rows x 128 B = 2 KiB, two such instructions):
+//     16-byte slot of (row r, chunk c) = 8*r + ((c + (r >> 1)) & 7).  The rotation
+//     is applied on the global side (lane 8r+j fetches chunk (j - (r >> 1)) & 7),
+//     so the LDS write stays linear in the lane id as the DMA requires, and the
+//     MFMA fragment read (lane l: row l & 15, chunk 4*half + (l >> 4)) finds the 16
+//     lanes of every K group in 16 different 16-byte bank groups: no bank
+//     conflicts, no padding.  (The intent of the reference's
+//     shared_memory_swizzle_coordinate, src/include/gemm_utils.cuh:15-20, which it
+//     applies on the read side only.)
+//   * Which K bytes a lane group holds does not matter as long as A and B agree:
+//     the contraction index is summed away.
+//   * LDS holds two stages (double buffer).
 //
 // Math
 //   * The B fragment is fed as the first MFMA operand and the A fragment as the
@@ -54,17 +60,29 @@ struct GemmArgs {
     int out_dtype;        // qgemm_dtype_t of C
     int per_matrix_scale; // multiply by as[0]*bs[0] in the epilogue
     int vec_store;        // C and ldc allow 16-byte (f32/i32) / 8-byte (16-bit) vector stores
+    int debug;            // reserved for measurement builds; the kernels ignore it
 };
 
 // How a stage travels from global memory to LDS.
 //   LOAD_DMA   buffer_load_dwordx4 ... lds: no VGPR staging, the wave only waits on vmcnt
 //   LOAD_VGPR  buffer_load_dwordx4 into registers during the MFMAs of the previous
-//              tile, ds_write_b128 afterwards; same LDS layout
+//              tile, ds_write_b128 afterwards; same addresses, same LDS layout
 enum Loader : int { LOAD_DMA = 0, LOAD_VGPR = 1 };
 
-template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int LOADER_ = LOAD_DMA>
+// How the K loop is scheduled.
+//   PIPE_SIMPLE    every wave: wait for tile k, barrier, start tile k+1, read fragments, MFMA.
+//   PIPE_PINGPONG  8 waves = 2 per SIMD.  Waves 0-3 and waves 4-7 run the same loop half a K
+//                  step apart: while one wave of a SIMD issues the MFMAs of tile k from
+//                  registers, its partner reads the fragments of its next tile from LDS and
+//                  starts the next global -> LDS copy.  The matrix core of every SIMD always
+//                  has one wave feeding it; barriers fall between the phases.
+enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1 };
+
+template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int LOADER_ = LOAD_DMA,
+          int PIPE_ = PIPE_SIMPLE>
 struct GemmCfg {
     static constexpr int LOADER = LOADER_;
+    static constexpr int PIPE = PIPE_;
     static constexpr int ARITH = ARITH_;
     static constexpr bool BLOCK_SCALE = BLOCK_SCALE_;
     static constexpr int BM = BM_, BN = BN_, BKB = 128;         // BKB: bytes of K per step
@@ -73,16 +91,18 @@ struct GemmCfg {
     static constexpr int THREADS = NW * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
     static constexpr int TM = WM / 16, TN = WN / 16;            // 16x16 MFMA tiles per wave
-    static constexpr int NA = BM / 16 * 2, NB = BN / 16 * 2;    // 1 KiB fragment blocks per stage
-    static constexpr int LPT = (NA + NB) / NW;                  // DMA instructions per wave per stage
-    static constexpr int STAGE_BYTES = (NA + NB) * 1024;
+    static constexpr int RBA = BM / 16, RBB = BN / 16;          // 2 KiB row blocks per stage
+    static constexpr int NLOAD = (RBA + RBB) * 2;               // 1 KiB load instructions per stage
+    static constexpr int LPT = NLOAD / NW;                      // ... per wave
+    static constexpr int STAGE_BYTES = (RBA + RBB) * 2048;
     static constexpr int NSTAGE = 2;
     static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
-    static_assert((NA + NB) % NW == 0, "fragment blocks must divide evenly over the waves");
+    static_assert(NLOAD % NW == 0, "load instructions must divide evenly over the waves");
     static_assert(!BLOCK_SCALE || ARITH == AR_F8, "block scales are defined for fp8 only");
     static_assert(!BLOCK_SCALE || (128 % WN == 0 || WN % 128 == 0), "wave tile must align with 128-wide scale blocks");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS is 160 KiB per CU");
+    static_assert(PIPE == PIPE_SIMPLE || (NW == 8 && LOADER == LOAD_DMA), "ping-pong needs 8 waves and the DMA loader");
 };
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -94,6 +114,19 @@ __device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t by
 
 // vmcnt(n) only (expcnt / lgkmcnt left at "no wait"), gfx9 encoding.
 __device__ inline constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+// lgkmcnt(0) only
+__device__ inline constexpr int waitcnt_lgkm0() { return 0xF | (3 << 14) | (0x7 << 4) | (0 << 8); }
+
+// s_barrier that nothing is scheduled across (MFMAs have no memory dependence the
+// compiler could see, so it would otherwise be free to move them into the other phase)
+__device__ inline void phase_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// 16-byte slot of (row r in 0..15, chunk c in 0..7) inside a 2 KiB row block
+__host__ __device__ inline constexpr int lds_slot(int r, int c) { return 8 * r + ((c + (r >> 1)) & 7); }
 
 template <int ARITH>
 struct AccT { typedef v4f type; };
@@ -146,7 +179,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 
     // ---- buffer resources: base at this tile's first row and first K byte; the
     // range ends with the last valid row, so rows past M / N read as out of
-    // range (never a fault) and only ever feed outputs that are not stored.
+    // range (never a fault; the DMA then writes zeros) and only ever feed outputs
+    // that are not stored.
     const uint32_t a_rows = p.M - row0 < (uint32_t)C::BM ? p.M - row0 : C::BM;
     const uint32_t b_rows = p.N - col0 < (uint32_t)C::BN ? p.N - col0 : C::BN;
     const uint32_t kbytes = (uint32_t)nk * C::BKB;
@@ -155,25 +189,27 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const __amdgpu_buffer_rsrc_t rb =
         make_rsrc(p.B + (size_t)col0 * p.ldb + (size_t)kbeg * C::BKB, (b_rows - 1) * p.ldb + kbytes);
 
-    // per-lane byte offsets of the LPT fragment blocks this wave fetches each stage
+    // ---- the LPT load instructions of this wave.  Instruction q (0 .. NLOAD-1) covers rows
+    // 8*(q & 1) .. +7 of row block q >> 1 and lands at stage + 1024*q.
     uint32_t voff[C::LPT];
     bool isA[C::LPT];
 #pragma unroll
     for (int i = 0; i < C::LPT; ++i) {
-        const int q = wave + i * C::NW;               // fragment block id within the stage
-        isA[i] = q < C::NA;
-        const int qq = isA[i] ? q : q - C::NA;
-        const uint32_t rowl = (qq >> 1) * 16 + (lane & 15);
-        voff[i] = rowl * (isA[i] ? p.lda : p.ldb) + (qq & 1) * 64 + (lane >> 4) * 16;
+        const int q = wave + i * C::NW;
+        const int rblk = q >> 1;
+        isA[i] = rblk < C::RBA;
+        const int r = 8 * (q & 1) + (lane >> 3);                     // row inside the row block
+        const int chunk = ((lane & 7) - (r >> 1)) & 7;               // rotation: see lds_slot
+        const uint32_t rowl = (isA[i] ? rblk : rblk - C::RBA) * 16 + r;
+        voff[i] = rowl * (isA[i] ? p.lda : p.ldb) + chunk * 16;
     }
 
-    auto issue_stage = [&](int kt) {
+    auto issue_stage = [&](int kt) {       // LOAD_DMA: global -> LDS
         char *stage = smem + (kt & 1) * C::STAGE_BYTES;
         const uint32_t soff = (uint32_t)kt * C::BKB;
 #pragma unroll
         for (int i = 0; i < C::LPT; ++i) {
-            const int q = wave + i * C::NW;
-            lds_void *dst = (lds_void *)(stage + q * 1024);
+            lds_void *dst = (lds_void *)(stage + (wave + i * C::NW) * 1024);
             if (isA[i])
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff[i], soff, 0, 0);
             else
@@ -189,7 +225,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             staged[i] = isA[i] ? __builtin_amdgcn_raw_buffer_load_b128(ra, voff[i], soff, 0)
                                : __builtin_amdgcn_raw_buffer_load_b128(rb, voff[i], soff, 0);
     };
-    auto commit_stage = [&](int kt) {      // LOAD_VGPR: registers -> LDS, same layout as the DMA path
+    auto commit_stage = [&](int kt) {      // LOAD_VGPR: registers -> LDS, where the DMA would have put them
         char *stage = smem + (kt & 1) * C::STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < C::LPT; ++i) *(v4i *)(stage + (wave + i * C::NW) * 1024 + lane * 16) = staged[i];
@@ -229,62 +265,130 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #pragma unroll
         for (int b = 0; b < C::TN; ++b) acc[a][b] = acc_t{0, 0, 0, 0};
 
-    const int lane_off = lane * 16;
-    const int a_frag0 = (wm * C::TM * 2) * 1024 + lane_off;
-    const int b_frag0 = (C::NA + wn * C::TN * 2) * 1024 + lane_off;
+    // ---- fragment addresses: lane l is row l & 15, K group l >> 4; its two 16-byte pieces
+    // of a K step are chunks (l >> 4) and 4 + (l >> 4) of that row
+    const int fr = lane & 15, fg = lane >> 4;
+    const int off0 = lds_slot(fr, fg) * 16, off1 = lds_slot(fr, 4 + fg) * 16;
+    const int a_blk0 = (wm * C::TM) * 2048;
+    const int b_blk0 = (C::RBA + wn * C::TN) * 2048;
+    auto frag_a = [&](const char *stage, int a, int half) {
+        return *(const v4i *)(stage + a_blk0 + a * 2048 + (half ? off1 : off0));
+    };
+    auto frag_b = [&](const char *stage, int b, int half) {
+        return *(const v4i *)(stage + b_blk0 + b * 2048 + (half ? off1 : off0));
+    };
 
     // ---- K loop
-    if (nk > 0) {
-        if constexpr (C::LOADER == LOAD_DMA) {
+    if constexpr (C::PIPE == PIPE_PINGPONG) {
+        // Waves 4-7 ("late" group) run one phase behind waves 0-3 ("early" group).  Phases:
+        //   memory : ds_read all fragments of tile kt into registers
+        //   compute: MFMAs of tile kt, operands all in registers
+        // In every even phase all waves start their part of the next tile's global -> LDS copy
+        // (early group at the top of its memory phase, late group at the top of its compute
+        // phase) and wait for it at the end of the following phase.  So a tile is complete one
+        // barrier before its first reader, and a stage is only overwritten one barrier after its
+        // last reader; the copy has one full K step to land.
+        const bool late = wave >= C::NW / 2;
+        v4i fa[C::TM][2], fb[C::TN][2];
+        if (nk > 0) {
             issue_stage(0);
-        } else {
-            fetch_stage(0);
-            commit_stage(0);
-        }
-        load_scales(0, as_nxt, bs_nxt);
-    }
-    for (int kt = 0; kt < nk; ++kt) {
-        if constexpr (C::LOADER == LOAD_DMA)
-            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // this wave's part of tile kt has landed
-        __syncthreads();                                 // ... and everybody else's; tile kt-1 is fully consumed
-        if constexpr (C::BLOCK_SCALE) {
-#pragma unroll
-            for (int a = 0; a < C::TM; ++a) as_cur[a] = as_nxt[a];
-#pragma unroll
-            for (int j = 0; j < NBS; ++j) bs_cur[j] = bs_nxt[j];
-        }
-        if (kt + 1 < nk) {
-            if constexpr (C::LOADER == LOAD_DMA) issue_stage(kt + 1);
-            else fetch_stage(kt + 1);
-            load_scales(kt + 1, as_nxt, bs_nxt);
-        }
-        const char *stage = smem + (kt & 1) * C::STAGE_BYTES;
-        v4i fa[C::TM][2];
-#pragma unroll
-        for (int a = 0; a < C::TM; ++a) {
-            fa[a][0] = *(const v4i *)(stage + a_frag0 + (a * 2 + 0) * 1024);
-            fa[a][1] = *(const v4i *)(stage + a_frag0 + (a * 2 + 1) * 1024);
-        }
-#pragma unroll
-        for (int b = 0; b < C::TN; ++b) {
-            const v4i fb0 = *(const v4i *)(stage + b_frag0 + (b * 2 + 0) * 1024);
-            const v4i fb1 = *(const v4i *)(stage + b_frag0 + (b * 2 + 1) * 1024);
-#pragma unroll
-            for (int a = 0; a < C::TM; ++a) {
-                if constexpr (C::BLOCK_SCALE) {
-                    // (P * as) * bs, then accumulate: hip_mix_gemm_kernel.cpp:241
-                    const v4f part = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                    const float sa = as_cur[a], sb = bs_cur[(b * 16) / 128];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[a][b][r] += (part[r] * sa) * sb;
-                } else {
-                    acc[a][b] = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], acc[a][b]);
-                }
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            phase_barrier();
+            if (late) {
+                if (nk > 1) issue_stage(1);
+                phase_barrier();
             }
         }
-        if constexpr (C::LOADER == LOAD_VGPR) {
-            // the other stage was last read in iteration kt-1, which every wave left before this one began
-            if (kt + 1 < nk) commit_stage(kt + 1);
+        for (int kt = 0; kt < nk; ++kt) {
+            // ---- memory phase
+            if constexpr (C::BLOCK_SCALE) load_scales(kt, as_cur, bs_cur);
+            if (!late && kt + 1 < nk) issue_stage(kt + 1);
+            const char *stage = smem + (kt & 1) * C::STAGE_BYTES;
+#pragma unroll
+            for (int a = 0; a < C::TM; ++a) {
+                fa[a][0] = frag_a(stage, a, 0);
+                fa[a][1] = frag_a(stage, a, 1);
+            }
+#pragma unroll
+            for (int b = 0; b < C::TN; ++b) {
+                fb[b][0] = frag_b(stage, b, 0);
+                fb[b][1] = frag_b(stage, b, 1);
+            }
+            __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());          // reads done before the stage may be refilled
+            if (late) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // copy started in the previous phase
+            phase_barrier();
+            // ---- compute phase
+            if (late && kt + 2 < nk) issue_stage(kt + 2);
+#pragma unroll
+            for (int b = 0; b < C::TN; ++b) {
+#pragma unroll
+                for (int a = 0; a < C::TM; ++a) {
+                    if constexpr (C::BLOCK_SCALE) {
+                        const v4f part = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                        const float sa = as_cur[a], sb = bs_cur[(b * 16) / 128];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[a][b][r] += (part[r] * sa) * sb;
+                    } else {
+                        acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                    }
+                }
+            }
+            if (!late) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // copy started in this wave's memory phase
+            if (!late || kt + 1 < nk) phase_barrier();
+        }
+    } else {
+        if (nk > 0) {
+            if constexpr (C::LOADER == LOAD_DMA) {
+                issue_stage(0);
+            } else {
+                fetch_stage(0);
+                commit_stage(0);
+            }
+            load_scales(0, as_nxt, bs_nxt);
+        }
+        for (int kt = 0; kt < nk; ++kt) {
+            if constexpr (C::LOADER == LOAD_DMA)
+                __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // this wave's part of tile kt has landed
+            __syncthreads();                                 // ... and everybody else's; tile kt-1 is fully consumed
+            if constexpr (C::BLOCK_SCALE) {
+#pragma unroll
+                for (int a = 0; a < C::TM; ++a) as_cur[a] = as_nxt[a];
+#pragma unroll
+                for (int j = 0; j < NBS; ++j) bs_cur[j] = bs_nxt[j];
+            }
+            if (kt + 1 < nk) {
+                if constexpr (C::LOADER == LOAD_DMA) issue_stage(kt + 1);
+                else fetch_stage(kt + 1);
+                load_scales(kt + 1, as_nxt, bs_nxt);
+            }
+            const char *stage = smem + (kt & 1) * C::STAGE_BYTES;
+            v4i fa[C::TM][2];
+#pragma unroll
+            for (int a = 0; a < C::TM; ++a) {
+                fa[a][0] = frag_a(stage, a, 0);
+                fa[a][1] = frag_a(stage, a, 1);
+            }
+#pragma unroll
+            for (int b = 0; b < C::TN; ++b) {
+                const v4i fb0 = frag_b(stage, b, 0);
+                const v4i fb1 = frag_b(stage, b, 1);
+#pragma unroll
+                for (int a = 0; a < C::TM; ++a) {
+                    if constexpr (C::BLOCK_SCALE) {
+                        // (P * as) * bs, then accumulate: hip_mix_gemm_kernel.cpp:241
+                        const v4f part = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                        const float sa = as_cur[a], sb = bs_cur[(b * 16) / 128];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[a][b][r] += (part[r] * sa) * sb;
+                    } else {
+                        acc[a][b] = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], acc[a][b]);
+                    }
+                }
+            }
+            if constexpr (C::LOADER == LOAD_VGPR) {
+                // the other stage was last read in iteration kt-1, which every wave left before this one began
+                if (kt + 1 < nk) commit_stage(kt + 1);
+            }
         }
     }
 

@@ -5,6 +5,7 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -30,6 +31,7 @@ struct Context {
     long force_config = -1;     // index into the variant table, -1 = heuristic
     long force_split = 0;       // 0 = heuristic
     long force_group_m = 0;     // 0 = default
+    long debug_flags = 0;       // GemmArgs::debug
     std::string last_config;
 };
 
@@ -51,6 +53,9 @@ int ensure_init_locked() {
     HIP_TRY(hipGetDeviceProperties(&prop, dev));
     g_ctx.device = dev;
     g_ctx.num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    // tuning knobs, also reachable through qgemm_set_option
+    if (const char *e = std::getenv("QGEMM_FORCE_CONFIG")) g_ctx.force_config = std::atol(e);
+    if (const char *e = std::getenv("QGEMM_GROUP_M")) g_ctx.force_group_m = std::atol(e);
     g_ctx.ready = true;
     return QGEMM_OK;
 }
@@ -124,20 +129,26 @@ bool mfma_shape_ok(const NtProblem &q) {
            q.M < ((size_t)1 << 31) && q.N < ((size_t)1 << 31) && q.ldc < ((size_t)1 << 32);
 }
 
-// Heuristic.  Pass 1: the largest tile that still gives every CU a workgroup.
-// Pass 2 (small problems): the shortest tile that covers min(M, 128) rows, so B
-// is streamed once, and the K split below supplies the parallelism.
+// Heuristic over the rows marked auto_ok.  Pass 1: the largest tile that still gives
+// every CU a workgroup.  Pass 2 (small problems): the shortest tile that covers
+// min(M, 128) rows, so B is streamed once, and the K split supplies the parallelism.
 int choose_variant(const Variant *tab, int count, size_t M, size_t N, int cus) {
     const size_t m16 = std::max<size_t>(16, (M + 15) / 16 * 16);
-    for (int i = 0; i < count; ++i) {
-        if (tab[i].loader != LOAD_DMA || (size_t)tab[i].bm > m16) continue;
-        const size_t tiles = ((M + tab[i].bm - 1) / tab[i].bm) * ((N + tab[i].bn - 1) / tab[i].bn);
-        if (tiles >= (size_t)cus) return i;
-    }
-    const size_t target = std::min<size_t>(m16, 128);
     int best = -1;
+    size_t best_area = 0;
     for (int i = 0; i < count; ++i) {
-        if (tab[i].loader != LOAD_DMA || (size_t)tab[i].bm < target) continue;
+        if (!tab[i].auto_ok || (size_t)tab[i].bm > m16) continue;
+        const size_t tiles = ((M + tab[i].bm - 1) / tab[i].bm) * ((N + tab[i].bn - 1) / tab[i].bn);
+        const size_t area = (size_t)tab[i].bm * tab[i].bn;
+        if (tiles >= (size_t)cus && area > best_area) {
+            best = i;
+            best_area = area;
+        }
+    }
+    if (best >= 0) return best;
+    const size_t target = std::min<size_t>(m16, 128);
+    for (int i = 0; i < count; ++i) {
+        if (!tab[i].auto_ok || (size_t)tab[i].bm < target) continue;
         if (best < 0 || tab[i].bm < tab[best].bm) best = i;
     }
     return best;
@@ -359,6 +370,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     if (!std::strcmp(key, "force_config")) g_ctx.force_config = value;
     else if (!std::strcmp(key, "force_split")) g_ctx.force_split = value;
     else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
+    else if (!std::strcmp(key, "debug_flags")) g_ctx.debug_flags = value;
     else return QGEMM_ERR_INVALID_ARG;
     return QGEMM_OK;
 }
@@ -718,6 +730,28 @@ QGEMM_EXPORT int qgemm_selftest_layouts(char *buf, size_t buflen) {
         (void)hipFree(dx);
         (void)hipFree(dy);
         (void)hipFree(dout);
+    }
+    // ---- which XCD does workgroup i land on?  The tile raster assumes i % 8.
+    {
+        const int nwg = 64;
+        void *dout = nullptr;
+        HIP_TRY(hipMalloc(&dout, nwg * 8));
+        hipLaunchKernelGGL(probe_xcc_kernel, dim3(nwg), dim3(64), 0, 0, (uint32_t *)dout);
+        HIP_TRY(hipGetLastError());
+        std::vector<uint32_t> h(nwg * 2);
+        HIP_TRY(hipMemcpy(h.data(), dout, nwg * 8, hipMemcpyDeviceToHost));
+        (void)hipFree(dout);
+        int round_robin = 0;
+        rep += "xcc of workgroups 0..31:";
+        for (int i = 0; i < nwg; ++i) {
+            if (i < 32) {
+                std::snprintf(line, sizeof(line), " %u", h[i * 2] & 15u);
+                rep += line;
+            }
+            round_robin += (int)(h[i * 2] & 15u) == i % kXcds;
+        }
+        std::snprintf(line, sizeof(line), "\nxcc round robin (wg %% 8): %d of %d workgroups\n", round_robin, nwg);
+        rep += line;
     }
     if (buf && buflen) std::snprintf(buf, buflen, "%s", rep.c_str());
     return all_ok ? QGEMM_OK : QGEMM_ERR_UNSUPPORTED;

@@ -44,4 +44,18 @@ __global__ void __launch_bounds__(64) probe_mfma_kernel(const char *x, const cha
 #endif
 }
 
+// Every workgroup records which XCD (XCC_ID hardware register) and CU it ran on.
+__global__ void __launch_bounds__(64) probe_xcc_kernel(uint32_t *out) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // s_getreg_b32 of HW_REG_XCC_ID (id 20), all 32 bits: XCC_ID in bits 3:0
+    const uint32_t xcc = __builtin_amdgcn_s_getreg((31 << 11) | 20);
+    // HW_REG_HW_ID (id 4): CU id in bits 11:8, SE id in bits 15:13 on gfx9
+    const uint32_t hw = __builtin_amdgcn_s_getreg((31 << 11) | 4);
+    if (threadIdx.x == 0) {
+        out[blockIdx.x * 2] = xcc;
+        out[blockIdx.x * 2 + 1] = hw;
+    }
+#endif
+}
+
 }  // namespace qgemm

@@ -12,6 +12,7 @@ struct Variant {
     int arith;
     bool block_scale;
     int bm, bn, threads, lds_bytes, loader;
+    bool auto_ok;   // the shape heuristic may pick this row (the others are reachable through force_config)
     hipError_t (*launch)(const GemmArgs &, uint32_t grid, hipStream_t);
 };
 
