@@ -23,7 +23,7 @@ static hipError_t launch_variant(const GemmArgs &a, uint32_t grid, hipStream_t s
     return hipGetLastError();
 }
 
-#define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP>
+#define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) == PIPE_PINGPONG>
 #define ROWP(NAME, BM, BN, WM_, WN_, LD, PP, AUTO)                                                    \
     {NAME, INST_ARITH, (bool)INST_BLOCK, BM, BN, CFG(BM, BN, WM_, WN_, LD, PP)::THREADS,             \
      CFG(BM, BN, WM_, WN_, LD, PP)::LDS_BYTES, LD, AUTO, &launch_variant<CFG(BM, BN, WM_, WN_, LD, PP)>}

@@ -38,6 +38,8 @@
 //     partial product of exactly one scale block, which is folded in with one
 //     FMA per element (hip_mix_gemm_kernel.cpp:231-244).
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace qgemm {
@@ -59,8 +61,8 @@ struct GemmArgs {
     uint32_t nb_max;      // ceil(N/128) - 1
     int out_dtype;        // qgemm_dtype_t of C
     int per_matrix_scale; // multiply by as[0]*bs[0] in the epilogue
-    int vec_store;        // C and ldc allow 16-byte (f32/i32) / 8-byte (16-bit) vector stores
-    int debug;            // reserved for measurement builds; the kernels ignore it
+    int vec_store;        // 0: scalar stores; 1: C and ldc allow 4-element vector stores; 2: also 16-byte row pieces
+    unsigned long long *dbg_cycles;   // DBG bit 3 builds only: per workgroup {start, loop start, loop end, end}
 };
 
 // How a stage travels from global memory to LDS.
@@ -78,11 +80,18 @@ enum Loader : int { LOAD_DMA = 0, LOAD_VGPR = 1 };
 //                  has one wave feeding it; barriers fall between the phases.
 enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1 };
 
+// TAIL_ (ping-pong): number of B-fragment columns of MFMAs a wave still issues after the
+// barrier that ends its compute phase, so the hand-over to its partner is hidden.
+// A3_   (ping-pong): A gets three LDS buffers and B two (exactly 160 KiB for 256 x 256):
+// the A copy of tile k+2 is started two K steps ahead and only the B half of a tile has to
+// land within one step.
 template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int LOADER_ = LOAD_DMA,
-          int PIPE_ = PIPE_SIMPLE>
+          int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false>
 struct GemmCfg {
     static constexpr int LOADER = LOADER_;
     static constexpr int PIPE = PIPE_;
+    static constexpr int TAIL = TAIL_;
+    static constexpr bool A3 = A3_;
     static constexpr int ARITH = ARITH_;
     static constexpr bool BLOCK_SCALE = BLOCK_SCALE_;
     static constexpr int BM = BM_, BN = BN_, BKB = 128;         // BKB: bytes of K per step
@@ -94,15 +103,19 @@ struct GemmCfg {
     static constexpr int RBA = BM / 16, RBB = BN / 16;          // 2 KiB row blocks per stage
     static constexpr int NLOAD = (RBA + RBB) * 2;               // 1 KiB load instructions per stage
     static constexpr int LPT = NLOAD / NW;                      // ... per wave
-    static constexpr int STAGE_BYTES = (RBA + RBB) * 2048;
-    static constexpr int NSTAGE = 2;
-    static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
+    static constexpr int A_BYTES = RBA * 2048, B_BYTES = RBB * 2048;
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int LPT_A = RBA * 2 / NW;                  // A load instructions per wave (ping-pong)
+    static constexpr int LDS_BYTES = A3 ? 3 * A_BYTES + 2 * B_BYTES : 2 * STAGE_BYTES;
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
     static_assert(NLOAD % NW == 0, "load instructions must divide evenly over the waves");
     static_assert(!BLOCK_SCALE || ARITH == AR_F8, "block scales are defined for fp8 only");
     static_assert(!BLOCK_SCALE || (128 % WN == 0 || WN % 128 == 0), "wave tile must align with 128-wide scale blocks");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS is 160 KiB per CU");
     static_assert(PIPE == PIPE_SIMPLE || (NW == 8 && LOADER == LOAD_DMA), "ping-pong needs 8 waves and the DMA loader");
+    static_assert(PIPE == PIPE_SIMPLE || (RBA * 2) % NW == 0, "ping-pong: A loads must divide evenly over the waves");
+    static_assert(PIPE == PIPE_PINGPONG || (TAIL == 0 && !A3), "TAIL and A3 belong to the ping-pong pipeline");
+    static_assert(TAIL >= 0 && TAIL < TN, "TAIL counts B-fragment columns");
 };
 
 typedef __attribute__((address_space(3))) void lds_void;
@@ -153,11 +166,15 @@ __device__ inline typename AccT<ARITH>::type mma128(v4i x0, v4i x1, v4i y0, v4i 
     }
 }
 
-template <class C>
+// DBG is a measurement aid for kernel bring-up (bit 0: skip the MFMAs, bit 1: skip the
+// global loads, bit 2: skip the fragment reads); the library only instantiates DBG = 0.
+template <class C, int DBG = 0>
 __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     typedef typename AccT<C::ARITH>::type acc_t;
+    unsigned long long dbg_t0 = 0, dbg_t1 = 0, dbg_t2 = 0;
+    if constexpr (DBG & 8) dbg_t0 = __builtin_readcyclecounter();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -279,62 +296,195 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     };
 
     // ---- K loop
+    if constexpr (DBG & 8) dbg_t1 = __builtin_readcyclecounter();
     if constexpr (C::PIPE == PIPE_PINGPONG) {
         // Waves 4-7 ("late" group) run one phase behind waves 0-3 ("early" group).  Phases:
         //   memory : ds_read all fragments of tile kt into registers
         //   compute: MFMAs of tile kt, operands all in registers
-        // In every even phase all waves start their part of the next tile's global -> LDS copy
-        // (early group at the top of its memory phase, late group at the top of its compute
-        // phase) and wait for it at the end of the following phase.  So a tile is complete one
-        // barrier before its first reader, and a stage is only overwritten one barrier after its
-        // last reader; the copy has one full K step to land.
-        const bool late = wave >= C::NW / 2;
+        // so whenever one wave of a SIMD is in its compute phase its partner is in its memory
+        // phase, and every phase boundary is one workgroup barrier ("slot" 2kt: early group reads
+        // tile kt, late group computes tile kt-1; slot 2kt+1: the other way round).
+        //
+        // Global -> LDS copies are issued one at a time between the ds_reads / MFMAs of a
+        // phase (a burst in front of the MFMAs would hold them back while the texture
+        // addresser works through the queue).  With A3: every wave issues its share of B(kt+1)
+        // in slot 2kt and of A(kt+2) in slot 2kt+1, and waits with vmcnt(LPT_A) at the end of
+        // every odd slot: that leaves only the A copy just issued, which has two more slots to
+        // land, in flight.  Without A3 both A(kt+1) and B(kt+1) go out in slot 2kt.
+        // A buffer is first read one barrier after the wait of its last copier, and is first
+        // overwritten one barrier after the lgkmcnt(0) of its last reader.
+        //
+        // The loop exists four times (early / late group, with / without the end-of-K guards)
+        // so that the steady state has no branches between the MFMAs.
+        constexpr int NA_BUF = C::A3 ? 3 : 2;
+        constexpr int B_BASE = NA_BUF * C::A_BYTES;
+        constexpr int LPT_A = C::LPT_A, LPT_B = C::LPT - C::LPT_A;
+        // instruction i < LPT_A of this wave belongs to A, the rest to B (RBA*2 % NW == 0)
+        auto issue_a1 = [&](int i, int kt, int buf) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                ra, (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024), 16, voff[i],
+                (uint32_t)kt * C::BKB, 0, 0);
+        };
+        auto issue_b1 = [&](int i, int kt) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                rb, (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (wave + i * C::NW) * 1024 - C::A_BYTES), 16,
+                voff[i], (uint32_t)kt * C::BKB, 0, 0);
+        };
+        auto next_buf = [&](int bufi) { return bufi + 1 == NA_BUF ? 0 : bufi + 1; };
+        // The copies of one slot as a numbered list 0 .. n-1, so a phase can issue them one by one.
+        //   even slot 2kt  : A3 ? B(kt+1)            : A(kt+1) then B(kt+1)
+        //   odd slot 2kt+1 : A3 ? A(kt+2) -> a_wr     : nothing
+        constexpr int N_EVEN = C::A3 ? LPT_B : C::LPT, N_ODD = C::A3 ? LPT_A : 0;
+        int a_wr = C::A3 ? 2 : 1;           // buffer the next A copy of this wave goes to
+        int a_rd = 0;                       // buffer holding A of the tile being read
+        // kt: tile the early group reads in this slot; guard: check the end of K
+        auto issue_even = [&](int j, int kt, bool guard) {
+            if constexpr (DBG & 2) return;
+            if (guard && kt + 1 >= nk) return;
+            if constexpr (C::A3) issue_b1(LPT_A + j, kt + 1);
+            else if (j < LPT_A) issue_a1(j, kt + 1, a_wr);
+            else issue_b1(j, kt + 1);
+        };
+        auto issue_odd = [&](int j, int kt, bool guard) {
+            if constexpr (DBG & 2) return;
+            if constexpr (C::A3) {
+                if (guard && kt + 2 >= nk) return;
+                issue_a1(j, kt + 2, a_wr);
+            }
+        };
         v4i fa[C::TM][2], fb[C::TN][2];
-        if (nk > 0) {
-            issue_stage(0);
-            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-            phase_barrier();
-            if (late) {
-                if (nk > 1) issue_stage(1);
-                phase_barrier();
+        constexpr int COLS_COPY = C::TN - C::TAIL;    // copies that can ride between the MFMA columns
+
+        // DBG bit 4: accumulate cycles per phase section (s_memtime, so only taken at points
+        // where no LDS read is outstanding)
+        unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, tprev = 0;
+        auto stamp = [&](int slot) {
+            if constexpr (DBG & 16) {
+                const unsigned long long t = __builtin_readcyclecounter();
+                ph[slot] += t - tprev;
+                tprev = t;
             }
-        }
-        for (int kt = 0; kt < nk; ++kt) {
-            // ---- memory phase
+        };
+
+        // one K step of one wave.  LATE / GUARD are std::integral_constant<bool>.
+        auto step = [&](int kt, auto late_tag, auto guard_tag) {
+            constexpr bool LATE = decltype(late_tag)::value, GUARD = decltype(guard_tag)::value;
+            // ---- memory phase (early: slot 2kt, even; late: slot 2kt+1, odd)
             if constexpr (C::BLOCK_SCALE) load_scales(kt, as_cur, bs_cur);
-            if (!late && kt + 1 < nk) issue_stage(kt + 1);
-            const char *stage = smem + (kt & 1) * C::STAGE_BYTES;
-#pragma unroll
-            for (int a = 0; a < C::TM; ++a) {
-                fa[a][0] = frag_a(stage, a, 0);
-                fa[a][1] = frag_a(stage, a, 1);
-            }
-#pragma unroll
-            for (int b = 0; b < C::TN; ++b) {
-                fb[b][0] = frag_b(stage, b, 0);
-                fb[b][1] = frag_b(stage, b, 1);
-            }
-            __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());          // reads done before the stage may be refilled
-            if (late) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // copy started in the previous phase
-            phase_barrier();
-            // ---- compute phase
-            if (late && kt + 2 < nk) issue_stage(kt + 2);
-#pragma unroll
-            for (int b = 0; b < C::TN; ++b) {
+            const char *sa_ = smem + a_rd * C::A_BYTES;
+            const char *sb_ = smem + B_BASE + (kt & 1) * C::B_BYTES - C::A_BYTES;   // frag_b adds RBA row blocks
+            constexpr int n_m = LATE ? N_ODD : N_EVEN;     // copies of this wave in this phase
+            if (!(DBG & 4) || kt == 0) {
 #pragma unroll
                 for (int a = 0; a < C::TM; ++a) {
-                    if constexpr (C::BLOCK_SCALE) {
-                        const v4f part = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                        const float sa = as_cur[a], sb = bs_cur[(b * 16) / 128];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[a][b][r] += (part[r] * sa) * sb;
-                    } else {
-                        acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                    if (a < n_m) {
+                        if constexpr (LATE) issue_odd(a, kt, GUARD);
+                        else issue_even(a, kt, GUARD);
                     }
+                    fa[a][0] = frag_a(sa_, a, 0);
+                    fa[a][1] = frag_a(sa_, a, 1);
+                }
+#pragma unroll
+                for (int b = 0; b < C::TN; ++b) {
+                    if (C::TM + b < n_m) {
+                        if constexpr (LATE) issue_odd(C::TM + b, kt, GUARD);
+                        else issue_even(C::TM + b, kt, GUARD);
+                    }
+                    fb[b][0] = frag_b(sb_, b, 0);
+                    fb[b][1] = frag_b(sb_, b, 1);
                 }
             }
-            if (!late) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // copy started in this wave's memory phase
-            if (!late || kt + 1 < nk) phase_barrier();
+            if constexpr (LATE ? (N_ODD > 0) : !C::A3) a_wr = next_buf(a_wr);
+            a_rd = next_buf(a_rd);
+            __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());   // reads done before the buffers may be refilled
+            stamp(0);
+            auto wait_copies = [&]() {   // end of an odd slot: all copies landed but (A3) the A copy just issued
+                __builtin_amdgcn_sched_barrier(0);   // stays behind the MFMAs of the phase
+                if (C::A3 && (!GUARD || kt + 2 < nk)) __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
+                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            };
+            if constexpr (LATE) wait_copies();
+            stamp(1);
+            phase_barrier();
+            stamp(2);
+            // ---- compute phase (early: slot 2kt+1, odd; late: slot 2kt+2, even)
+            constexpr int n_c = LATE ? N_EVEN : N_ODD;
+            const int kt_slot = LATE ? kt + 1 : kt;
+#pragma unroll
+            for (int j = COLS_COPY; j < n_c; ++j) {        // copies that do not fit between the columns
+                if constexpr (LATE) issue_even(j, kt_slot, GUARD);
+                else issue_odd(j, kt_slot, GUARD);
+            }
+            auto mfma_cols = [&](int b0, int b1, int ncopy) {
+#pragma unroll
+                for (int b = b0; b < b1; ++b) {
+                    if (b < ncopy) {              // one copy in front of each of the first columns
+                        if constexpr (LATE) issue_even(b, kt_slot, GUARD);
+                        else issue_odd(b, kt_slot, GUARD);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    if constexpr (DBG & 1) continue;
+#pragma unroll
+                    for (int a = 0; a < C::TM; ++a) {
+                        if constexpr (C::BLOCK_SCALE) {
+                            const v4f part =
+                                mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                            const float sa = as_cur[a], sb = bs_cur[(b * 16) / 128];
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) acc[a][b][r] += (part[r] * sa) * sb;
+                        } else {
+                            acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                        }
+                    }
+                }
+            };
+            mfma_cols(0, C::TN - C::TAIL, n_c < COLS_COPY ? n_c : COLS_COPY);
+            if constexpr (LATE ? !C::A3 : (N_ODD > 0)) a_wr = next_buf(a_wr);
+            stamp(3);
+            if constexpr (!LATE) wait_copies();
+            stamp(4);
+            if (!LATE || !GUARD || kt + 1 < nk) phase_barrier();
+            stamp(5);
+            mfma_cols(C::TN - C::TAIL, C::TN, 0);
+        };
+
+        if (nk > 0) {
+#pragma unroll
+            for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
+#pragma unroll
+            for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 0);
+            if (C::A3 && nk > 1) {
+#pragma unroll
+                for (int i = 0; i < LPT_A; ++i) issue_a1(i, 1, 1);
+                __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
+            } else {
+                __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            }
+            phase_barrier();
+        }
+        typedef std::integral_constant<bool, true> yes_t;
+        typedef std::integral_constant<bool, false> no_t;
+        const int nk_fast = nk > 3 ? nk - 3 : 0;    // steps that cannot touch the end of K
+        if (wave >= C::NW / 2) {
+            if (nk > 0) {                   // slot 0 of the late group: only its copies
+#pragma unroll
+                for (int j = 0; j < N_EVEN; ++j) issue_even(j, 0, true);
+                if (!C::A3) a_wr = next_buf(a_wr);
+                phase_barrier();
+            }
+            if constexpr (DBG & 16) tprev = __builtin_readcyclecounter();
+            int kt = 0;
+            for (; kt < nk_fast; ++kt) step(kt, yes_t{}, no_t{});
+            for (; kt < nk; ++kt) step(kt, yes_t{}, yes_t{});
+        } else {
+            if constexpr (DBG & 16) tprev = __builtin_readcyclecounter();
+            int kt = 0;
+            for (; kt < nk_fast; ++kt) step(kt, no_t{}, no_t{});
+            for (; kt < nk; ++kt) step(kt, no_t{}, yes_t{});
+        }
+        if constexpr (DBG & 16) {
+            if (lane == 0)
+                for (int i = 0; i < 6; ++i) p.dbg_cycles[((size_t)blockIdx.x * C::NW + wave) * 8 + i] = ph[i];
         }
     } else {
         if (nk > 0) {
@@ -392,10 +542,68 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     }
 
+    if constexpr (DBG & 8) dbg_t2 = __builtin_readcyclecounter();
     // ---- epilogue: lane holds C[m][n0 .. n0+3] of every 16x16 tile
     float scale = 1.0f;
     if (p.per_matrix_scale) scale = p.as[0] * p.bs[0];
     char *Cz = p.C + (size_t)z * p.split_stride * dtype_bytes(p.out_dtype);
+
+    // Fast path: the wave tile lies inside C and rows of C are 16-byte aligned.  The accumulator
+    // layout (adjacent lanes = adjacent rows of C) would make every lane of a store its own
+    // request; so each 16-row slab goes through this wave's private LDS scratch and leaves as
+    // whole 16-byte-per-lane rows.  LDS is free here: in the ping-pong pipeline every wave is
+    // past the barrier that follows the last fragment read of both groups; the simple pipeline
+    // needs one more barrier.
+    constexpr int EPI_PITCH = C::WN * 4 + 16;
+    constexpr int EPI_BYTES = 16 * EPI_PITCH;
+    constexpr bool EPI_FITS = C::NW * EPI_BYTES <= C::LDS_BYTES;
+    if constexpr (C::PIPE == PIPE_SIMPLE && EPI_FITS) __syncthreads();
+    const bool wave_tile_full = row0 + wm * C::WM + C::WM <= p.M && col0 + wn * C::WN + C::WN <= p.N;
+    if (EPI_FITS && p.vec_store == 2 && wave_tile_full) {
+        char *scratch = smem + wave * EPI_BYTES;
+        const int es = dtype_bytes(p.out_dtype);
+        const int lanes_per_row = C::WN * es / 16, rows_per_pass = 64 / lanes_per_row;
+        const int rd_row = lane / lanes_per_row, rd_col = (lane % lanes_per_row) * 16;
+        char *wr = scratch + (lane & 15) * EPI_PITCH + (lane >> 4) * 4 * es;
+        const size_t c_row_bytes = (size_t)p.ldc * es;
+        char *cbase = Cz + ((size_t)(row0 + wm * C::WM) * p.ldc + col0 + wn * C::WN) * es + rd_col;
+#pragma unroll
+        for (int a = 0; a < C::TM; ++a) {
+#pragma unroll
+            for (int b = 0; b < C::TN; ++b) {
+                if (es == 4) {
+                    if (p.out_dtype == QGEMM_DT_I32) {
+                        *(acc_t *)(wr + b * 16 * 4) = acc[a][b];
+                    } else {
+                        v4f v;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) v[r] = (float)acc[a][b][r] * scale;
+                        *(v4f *)(wr + b * 16 * 4) = v;
+                    }
+                } else {
+                    us4 h;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float v = (float)acc[a][b][r] * scale;
+                        h[r] = p.out_dtype == QGEMM_DT_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+                    }
+                    *(us4 *)(wr + b * 16 * 2) = h;
+                }
+            }
+            for (int row = rd_row; row < 16; row += rows_per_pass) {
+                const v4i v = *(const v4i *)(scratch + row * EPI_PITCH + rd_col);
+                *(v4i *)(cbase + (size_t)(a * 16 + row) * c_row_bytes) = v;
+            }
+        }
+        if constexpr (DBG & 8) {
+            const unsigned long long t3 = __builtin_readcyclecounter();
+            if (lane == 0 && !(DBG & 16)) {
+                unsigned long long *o = p.dbg_cycles + ((size_t)blockIdx.x * C::NW + wave) * 4;
+                o[0] = dbg_t0; o[1] = dbg_t1; o[2] = dbg_t2; o[3] = t3;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int a = 0; a < C::TM; ++a) {
         const uint32_t m = row0 + wm * C::WM + a * 16 + (lane & 15);
@@ -436,6 +644,13 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     for (int r = 0; r < 4; ++r)
                         if (n + r < p.N) dst[r] = h[r];
             }
+        }
+    }
+    if constexpr (DBG & 8) {
+        const unsigned long long t3 = __builtin_readcyclecounter();
+        if (lane == 0) {
+            unsigned long long *o = p.dbg_cycles + ((size_t)blockIdx.x * C::NW + wave) * 4;
+            if constexpr (!(DBG & 16)) { o[0] = dbg_t0; o[1] = dbg_t1; o[2] = dbg_t2; o[3] = t3; }
         }
     }
 #endif

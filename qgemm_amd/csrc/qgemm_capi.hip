@@ -223,6 +223,7 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
         const int ob = dtype_bytes(q.out_dtype);
         const int vec = ob == 4 ? 16 : 8;
         a.vec_store = ((uintptr_t)q.C % vec == 0) && ((q.ldc * ob) % vec == 0);
+        if (a.vec_store && (uintptr_t)q.C % 16 == 0 && (q.ldc * ob) % 16 == 0) a.vec_store = 2;
         hipError_t e = v.launch(a, (uint32_t)pl.tiles, stream);
         g_ctx.last_config = v.name;
         return e == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
@@ -235,7 +236,7 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
     a.split_stride = plane;
     a.out_dtype = i32_acc ? QGEMM_DT_I32 : QGEMM_DT_F32;
     a.per_matrix_scale = 0;
-    a.vec_store = (q.N % 4 == 0);
+    a.vec_store = (q.N % 4 == 0) ? 2 : 0;   // workspace planes are 256-byte aligned, 4-byte elements
     hipError_t e = v.launch(a, (uint32_t)(pl.tiles * a.nsplit), stream);
     if (e != hipSuccess) return QGEMM_ERR_LAUNCH;
 
