@@ -134,10 +134,11 @@ bool mfma_shape_ok(const NtProblem &q) {
 // min(M, 128) rows, so B is streamed once, and the K split supplies the parallelism.
 int choose_variant(const Variant *tab, int count, size_t M, size_t N, int cus) {
     const size_t m16 = std::max<size_t>(16, (M + 15) / 16 * 16);
+    const size_t target = std::min<size_t>(m16, 128);   // shorter tiles would stream B more than once
     int best = -1;
     size_t best_area = 0;
     for (int i = 0; i < count; ++i) {
-        if (!tab[i].auto_ok || (size_t)tab[i].bm > m16) continue;
+        if (!tab[i].auto_ok || (size_t)tab[i].bm > m16 || (size_t)tab[i].bm < target) continue;
         const size_t tiles = ((M + tab[i].bm - 1) / tab[i].bm) * ((N + tab[i].bn - 1) / tab[i].bn);
         const size_t area = (size_t)tab[i].bm * tab[i].bn;
         if (tiles >= (size_t)cus && area > best_area) {
@@ -146,7 +147,6 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, int cus) {
         }
     }
     if (best >= 0) return best;
-    const size_t target = std::min<size_t>(m16, 128);
     for (int i = 0; i < count; ++i) {
         if (!tab[i].auto_ok || (size_t)tab[i].bm < target) continue;
         if (best < 0 || tab[i].bm < tab[best].bm) best = i;

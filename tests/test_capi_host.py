@@ -1,0 +1,90 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol
+include/qgemm.h declares, validates arguments before touching a device, and its tile
+raster is a bijection."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import qgemm_amd as Q
+from qgemm_amd import lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "qgemm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(qgemm_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = L.load_library()
+    names = _declared_symbols()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/qgemm.h but not exported"
+        assert n in L.SIGNATURES, f"{n} has no ctypes signature in qgemm_amd/lib.py"
+    # and nothing in the binding that the header does not declare
+    assert sorted(L.SIGNATURES) == names
+
+
+def test_status_strings():
+    lib = L.load_library()
+    assert lib.qgemm_status_string(0) == b"ok"
+    # the reference's throw texts, hip_mix_gemm_kernel.cpp:460,485,503
+    assert b"BLOCK_TILE_SIZE_M" in lib.qgemm_status_string(6)
+    assert b"BLOCK_TILE_SIZE_N" in lib.qgemm_status_string(7)
+    assert b"BLOCK_TILE_SIZE_K" in lib.qgemm_status_string(8)
+    assert lib.qgemm_status_string(12345) == b"unknown status"
+
+
+def test_argument_validation_needs_no_device():
+    lib = L.load_library()
+    one = C.c_void_p(16)
+    # unknown dtype / dtype pair
+    assert lib.qgemm_gemm(99, 0, 1, one, 16, one, 16, one, 16, 16, 16, 16, None) == 2
+    assert lib.qgemm_gemm(Q.DT_BF16, Q.DT_I32, 1, one, 16, one, 16, one, 16, 16, 16, 16, None) == 2
+    # bad layout enum, leading dimension smaller than the row
+    assert lib.qgemm_gemm(Q.DT_BF16, Q.DT_F32, 7, one, 16, one, 16, one, 16, 16, 16, 16, None) == 1
+    # scaled: only int8 / fp8 inputs; block scales only for fp8; reference layout checks divisibility first
+    assert lib.qgemm_scaled_gemm(Q.DT_BF16, Q.DT_F32, 1, 0, one, one, one, one, one, 16, 16, 16, 16, 0, None) == 2
+    assert lib.qgemm_scaled_gemm(Q.DT_I8, Q.DT_F32, 2, 0, one, one, one, one, one, 16, 16, 16, 16, 0, None) == 2
+    assert lib.qgemm_scaled_gemm(Q.DT_F8E4M3, Q.DT_BF16, 2, 1, one, one, one, one, one, 64, 48, 64, 128, 0, None) == 6
+    assert lib.qgemm_scaled_gemm(Q.DT_F8E4M3, Q.DT_BF16, 2, 1, one, one, one, one, one, 48, 64, 48, 128, 0, None) == 7
+    assert lib.qgemm_scaled_gemm(Q.DT_F8E4M3, Q.DT_BF16, 2, 1, one, one, one, one, one, 64, 64, 64, 80, 0, None) == 8
+    assert lib.qgemm_scaled_gemm(Q.DT_F8E4M3, Q.DT_BF16, 2, 0, one, one, one, one, one, 64, 64, 64, 128, -1, None) == 1
+    assert lib.qgemm_transpose(3, one, one, 4, 4, None) == 2
+    assert lib.qgemm_set_option(b"no_such_option", 1) == 1
+    if lib.qgemm_device_count() == 0:
+        assert lib.qgemm_init() == 3          # QGEMM_ERR_NO_DEVICE: loud, no CPU fallback
+        assert lib.qgemm_gemm(Q.DT_BF16, Q.DT_F32, 1, one, 16, one, 16, one, 16, 16, 16, 16, None) == 3
+
+
+def test_python_ops_refuse_host_tensors():
+    import torch
+    a = torch.zeros((16, 16), dtype=torch.int8)
+    with pytest.raises(ValueError):
+        Q.int8_mm(a, a, torch.ones(1), torch.ones(1), torch.zeros((16, 16), dtype=torch.int32))
+
+
+@pytest.mark.parametrize("tiles_m,tiles_n", [(32, 32), (1, 1), (1, 9), (7, 5), (24, 18), (3, 100), (48, 36), (2, 7)])
+@pytest.mark.parametrize("group", [1, 4, 8, 16])
+def test_tile_raster_is_a_bijection(tiles_m, tiles_n, group):
+    """XCD remap + GROUP_M raster (replaces sm89_gemm_kernel_v3.cu:169-183): every tile exactly once."""
+    total = tiles_m * tiles_n
+    seen = {Q.tile_map(w, tiles_m, tiles_n, group) for w in range(total)}
+    assert seen == {(i, j) for i in range(tiles_m) for j in range(tiles_n)}
+    with pytest.raises(Q.QgemmError):
+        Q.tile_map(total, tiles_m, tiles_n, group)
+
+
+def test_tile_raster_keeps_an_xcd_on_a_compact_cluster():
+    """Workgroups w, w+8, w+16, .. share an XCD (and its L2): their first 32 tiles must reuse few A / B panels."""
+    tiles_m = tiles_n = 32
+    for xcd in range(8):
+        first = [Q.tile_map(xcd + 8 * i, tiles_m, tiles_n, 8) for i in range(32)]
+        rows = {t[0] for t in first}
+        cols = {t[1] for t in first}
+        assert len(rows) + len(cols) <= 12      # 8 x 4 cluster: 12 panels for 32 tiles

@@ -1,0 +1,148 @@
+"""The five BASELINE configurations at their full sizes.
+
+Where the CPU oracle cannot finish the whole problem in seconds, the check is the oracle on
+sampled full rows and full columns of C, plus size-independent properties of the whole matrix:
+int32 results are identical bit for bit between two different tile configurations; scaling an
+operand's scale by a power of two scales C exactly; a K split leaves int32 results unchanged."""
+import numpy as np
+import pytest
+import torch
+
+import qgemm_amd as Q
+from oracle import cpu_ref as R
+from tests.util import assert_close, dev, fp8_tensor, host, say, scalar
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _reset_options():
+    yield
+    Q.set_option("force_config", -1)
+    Q.set_option("force_split", 0)
+
+
+def _sample(n, count, seed):
+    return np.sort(np.random.default_rng(seed).choice(n, size=count, replace=False))
+
+
+def test_cfg1_fp16_1024_b_stored_transposed():
+    """FP16 GEMM M=N=K=1024, A MxK, B stored NxK, uniform[-1,1], fp32 accumulate, fp16 out; whole matrix."""
+    M = N = K = 1024
+    say("cfg1 fp16 1024^3")
+    ha, hb = R.encode_f16(R.fill_uniform((M, K), 42)), R.encode_f16(R.fill_uniform((N, K), 43))
+    ref = R.gemm_f32acc(R.decode_f16(ha), R.decode_f16(hb))
+    a, b = dev(ha.view(np.int16)).view(torch.float16), dev(hb.view(np.int16)).view(torch.float16)
+    c = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    Q.gemm(a, b, c, "nk")
+    # fp16 output: half an ulp (2^-11 relative) on top of accumulation-order slack
+    assert_close(host(c).astype(np.float32), ref, rtol=2.0 ** -10, atol=2e-3, what=Q.last_config())
+
+
+def test_cfg2_int8_4096_bit_exact():
+    """INT8 per-matrix 4096^3: int32 accumulators bit-exact on 64 full rows and 64 full columns against the
+    oracle, identical over the whole matrix between two tile configurations and a K split; fp32 output equals
+    float(acc) * (sA * sB) bit for bit."""
+    M = N = K = 4096
+    say("cfg2 int8 4096^3")
+    qa, sa = R.quantize_int8(R.fill_normal((M, K), 42))
+    qb, sb = R.quantize_int8(R.fill_normal((N, K), 43))
+    da, db_ = dev(qa), dev(qb)
+    c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    Q.int8_mm(da, db_, scalar(sa), scalar(sb), c)
+    name0 = Q.last_config()
+    got = host(c)
+    rows, cols = _sample(M, 64, 1), _sample(N, 64, 2)
+    assert np.array_equal(got[rows], R.gemm_i8_i32(qa[rows], qb)), name0
+    assert np.array_equal(got[:, cols], R.gemm_i8_i32(qa, qb[cols])), name0
+    # another tile configuration and a K split: the same integers everywhere
+    Q.set_option("force_config", 2)
+    c2 = torch.zeros_like(c)
+    Q.int8_mm(da, db_, scalar(sa), scalar(sb), c2)
+    assert Q.last_config() != name0 and torch.equal(c, c2)
+    Q.set_option("force_config", -1)
+    c3 = torch.zeros_like(c)
+    Q.int8_mm(da, db_, scalar(sa), scalar(sb), c3, split_k=4)
+    assert "splitk" in Q.last_config() and torch.equal(c, c3)
+    cf = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.int8_mm(da, db_, scalar(sa), scalar(sb), cf)
+    assert np.array_equal(host(cf), R.scale_i32_to_f32(got, sa, sb))
+
+
+def test_cfg3_fp8_per_matrix_8192():
+    """FP8 e4m3 per-matrix 8192^3, bf16 out: rtol 2e-2 / atol 1e-2 against the fp32-accumulate oracle on 32 full
+    rows and 32 full columns; doubling sA doubles every output exactly; two tile configurations agree to bf16
+    rounding."""
+    M = N = K = 8192
+    say("cfg3 fp8 8192^3")
+    qa, sa = R.quantize_fp8(R.fill_normal((M, K), 42))
+    qb, sb = R.quantize_fp8(R.fill_normal((N, K), 43))
+    assert R.decode_fp8(qa).__abs__().max() == 448.0          # max|x| maps to 448
+    da, db_ = fp8_tensor(qa), fp8_tensor(qb)
+    c = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(da, db_, scalar(sa), scalar(sb), c, M, N, K, Q.SCALE_PER_MATRIX)
+    name0 = Q.last_config()
+    got = host(c)
+    rows, cols = _sample(M, 32, 3), _sample(N, 32, 4)
+    fb = R.decode_fp8(qb)
+    assert_close(got[rows], R.gemm_f32acc(R.decode_fp8(qa[rows]), fb) * np.float32(sa * sb), what=name0 + " rows")
+    del fb
+    assert_close(got[:, cols], R.gemm_f32acc(R.decode_fp8(qa), R.decode_fp8(qb[cols])) * np.float32(sa * sb),
+                 what=name0 + " cols")
+    c2 = torch.zeros_like(c)
+    Q.scaled_gemm(da, db_, scalar(2 * sa), scalar(sb), c2, M, N, K, Q.SCALE_PER_MATRIX)
+    assert torch.equal(c2.float(), 2 * c.float())              # power-of-two scale: exact
+    Q.set_option("force_config", 0)
+    c3 = torch.zeros_like(c)
+    Q.scaled_gemm(da, db_, scalar(sa), scalar(sb), c3, M, N, K, Q.SCALE_PER_MATRIX)
+    assert Q.last_config() != name0
+    # same products, different fp32 summation order: at most one bf16 ulp apart
+    assert torch.all((c3.float() - c.float()).abs() <= 2.0 ** -7 * c.float().abs() + 1e-3)
+
+
+def test_cfg4_fp8_block_scaled_6144x4608x7168():
+    """FP8 block-scaled M=6144 N=4608 K=7168: a_scale [M, K/128], b_scale [N/128, K/128] uniform[0.5, 2], bf16
+    out; oracle (per-128-block partial, then (P*as)*bs) on 24 full rows and 24 full columns."""
+    M, N, K = 6144, 4608, 7168
+    say("cfg4 fp8 block-scaled")
+    qa, _ = R.quantize_fp8(R.fill_normal((M, K), 42))
+    qb, _ = R.quantize_fp8(R.fill_normal((N, K), 43))
+    # scales uniform[0.5, 2], times the 1/448 a quantiser would have produced, so C is O(sqrt(K))
+    as_ = R.fill_uniform((M, K // 128), 44, 0.5, 2.0) * np.float32(5.0 / 448.0)
+    bs = R.fill_uniform((N // 128, K // 128), 45, 0.5, 2.0) * np.float32(5.0 / 448.0)
+    c = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
+    got = host(c)
+    rows, cols = _sample(M, 24, 5), _sample(N, 24, 6)
+    fb = R.decode_fp8(qb)
+    assert_close(got[rows], R.gemm_fp8_block(R.decode_fp8(qa[rows]), fb, as_[rows], bs), what=Q.last_config())
+    del fb
+    # a column sample needs the b_scale row of each sampled column's 128-block: evaluate per block
+    fa = R.decode_fp8(qa)
+    for nb in np.unique(cols // 128):
+        sel = cols[cols // 128 == nb]
+        ref = R.gemm_fp8_block(fa, R.decode_fp8(qb[sel]), as_, bs[nb:nb + 1])
+        assert_close(got[:, sel], ref, what=f"{Q.last_config()} cols of block {nb}")
+
+
+@pytest.mark.parametrize("M", [16, 64, 128])
+def test_cfg5_skinny_split_k(M):
+    """Skinny split-K, N=7168, K=2048, int8 (bit-exact) and fp8 (tolerance) with per-matrix scales; whole matrix."""
+    N, K = 7168, 2048
+    say("cfg5 skinny", M)
+    qa, sa = R.quantize_int8(R.fill_normal((M, K), 42))
+    qb, sb = R.quantize_int8(R.fill_normal((N, K), 43))
+    acc = R.gemm_i8_i32(qa, qb)
+    c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), c)
+    assert "splitk" in Q.last_config(), Q.last_config()       # the heuristic splits K for this shape
+    assert np.array_equal(host(c), acc)
+    cf = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), cf)
+    assert np.array_equal(host(cf), R.scale_i32_to_f32(acc, sa, sb))
+    fa, ta = R.quantize_fp8(R.fill_normal((M, K), 44))
+    fb, tb = R.quantize_fp8(R.fill_normal((N, K), 45))
+    cb = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(fa), fp8_tensor(fb), scalar(ta), scalar(tb), cb, M, N, K, Q.SCALE_PER_MATRIX)
+    assert_close(host(cb), R.gemm_f32acc(R.decode_fp8(fa), R.decode_fp8(fb)) * np.float32(ta * tb),
+                 what=Q.last_config())
