@@ -29,9 +29,7 @@ static hipError_t launch_variant(const GemmArgs &a, uint32_t grid, hipStream_t s
      CFG(BM, BN, WM_, WN_, LD, PP)::LDS_BYTES, LD, AUTO, &launch_variant<CFG(BM, BN, WM_, WN_, LD, PP)>}
 #define ROW(NAME, BM, BN, WM_, WN_, LD, AUTO) ROWP(NAME, BM, BN, WM_, WN_, LD, PIPE_SIMPLE, AUTO)
 
-// Order matters: the heuristic walks the auto rows from large to small tiles, and
-// force_config indexes this table.  Block-scaled builds keep the simple pipeline for the
-// 256x256 tile (the in-loop rescale does not fit the ping-pong register budget).
+// force_config indexes this table; the heuristic only considers the rows marked auto.
 static const Variant kTable[] = {
     ROW("256x256_w2x4_dma", 256, 256, 2, 4, LOAD_DMA, false),
     ROW("256x128_w2x2_dma", 256, 128, 2, 2, LOAD_DMA, false),
@@ -39,10 +37,10 @@ static const Variant kTable[] = {
     ROW("64x128_w1x4_dma", 64, 128, 1, 4, LOAD_DMA, true),
     ROW("32x128_w1x4_dma", 32, 128, 1, 4, LOAD_DMA, true),
     ROW("16x128_w1x2_dma", 16, 128, 1, 2, LOAD_DMA, true),
-    ROW("256x256_w2x4_vgpr", 256, 256, 2, 4, LOAD_VGPR, (bool)INST_BLOCK),
+    ROW("256x256_w2x4_vgpr", 256, 256, 2, 4, LOAD_VGPR, false),
     ROW("128x128_w2x2_vgpr", 128, 128, 2, 2, LOAD_VGPR, false),
     ROW("32x128_w1x4_vgpr", 32, 128, 1, 4, LOAD_VGPR, false),
-    ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, !(bool)INST_BLOCK),
+    ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, true),
     ROWP("256x256_w2x4_pingpong", 256, 256, 2, 4, LOAD_DMA, PIPE_PINGPONG, false),
 };
 

@@ -206,41 +206,39 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const __amdgpu_buffer_rsrc_t rb =
         make_rsrc(p.B + (size_t)col0 * p.ldb + (size_t)kbeg * C::BKB, (b_rows - 1) * p.ldb + kbytes);
 
-    // ---- the LPT load instructions of this wave.  Instruction q (0 .. NLOAD-1) covers rows
-    // 8*(q & 1) .. +7 of row block q >> 1 and lands at stage + 1024*q.
-    uint32_t voff[C::LPT];
-    bool isA[C::LPT];
-#pragma unroll
-    for (int i = 0; i < C::LPT; ++i) {
-        const int q = wave + i * C::NW;
-        const int rblk = q >> 1;
-        isA[i] = rblk < C::RBA;
-        const int r = 8 * (q & 1) + (lane >> 3);                     // row inside the row block
-        const int chunk = ((lane & 7) - (r >> 1)) & 7;               // rotation: see lds_slot
-        const uint32_t rowl = (isA[i] ? rblk : rblk - C::RBA) * 16 + r;
-        voff[i] = rowl * (isA[i] ? p.lda : p.ldb) + chunk * 16;
-    }
+    // ---- the LPT load instructions of this wave.  Instruction q = wave + i*NW (0 .. NLOAD-1) covers
+    // rows 8*(q & 1) .. +7 of row block q >> 1 and lands at stage + 1024*q.  With NW even, q & 1 =
+    // wave & 1 for every i, so the per-lane part of the address (row inside the block, rotated
+    // chunk) is the same for all of them: one VGPR per operand; the row block goes into the scalar
+    // offset of the instruction, which the buffer range check includes.
+    static_assert(C::NW % 2 == 0 && C::RBA % (C::NW / 2) == 0, "A / B split of the loads must not depend on the wave");
+    constexpr int LPT_A0 = C::LPT_A;                                    // loads i < LPT_A0 fetch A, the rest B
+    const int ld_r = 8 * (wave & 1) + (lane >> 3);                      // row inside the row block
+    const int ld_chunk = ((lane & 7) - (ld_r >> 1)) & 7;                // rotation: see lds_slot
+    const uint32_t voff_a = ld_r * p.lda + ld_chunk * 16, voff_b = ld_r * p.ldb + ld_chunk * 16;
+    auto load_soff = [&](int i, int kt) -> uint32_t {                   // scalar: row block + K step
+        const uint32_t blk = (wave >> 1) + (i < LPT_A0 ? i : i - LPT_A0) * (C::NW / 2);
+        return blk * 16 * (i < LPT_A0 ? p.lda : p.ldb) + (uint32_t)kt * C::BKB;
+    };
 
     auto issue_stage = [&](int kt) {       // LOAD_DMA: global -> LDS
         char *stage = smem + (kt & 1) * C::STAGE_BYTES;
-        const uint32_t soff = (uint32_t)kt * C::BKB;
 #pragma unroll
         for (int i = 0; i < C::LPT; ++i) {
             lds_void *dst = (lds_void *)(stage + (wave + i * C::NW) * 1024);
-            if (isA[i])
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff[i], soff, 0, 0);
+            if (i < LPT_A0)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, load_soff(i, kt), 0, 0);
             else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff[i], soff, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, load_soff(i, kt), 0, 0);
         }
     };
 
     v4i staged[C::LOADER == LOAD_VGPR ? C::LPT : 1];
     auto fetch_stage = [&](int kt) {       // LOAD_VGPR: global -> registers
-        const uint32_t soff = (uint32_t)kt * C::BKB;
 #pragma unroll
         for (int i = 0; i < C::LPT; ++i)
-            staged[i] = isA[i] ? __builtin_amdgcn_raw_buffer_load_b128(ra, voff[i], soff, 0)
-                               : __builtin_amdgcn_raw_buffer_load_b128(rb, voff[i], soff, 0);
+            staged[i] = i < LPT_A0 ? __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a, load_soff(i, kt), 0)
+                                   : __builtin_amdgcn_raw_buffer_load_b128(rb, voff_b, load_soff(i, kt), 0);
     };
     auto commit_stage = [&](int kt) {      // LOAD_VGPR: registers -> LDS, where the DMA would have put them
         char *stage = smem + (kt & 1) * C::STAGE_BYTES;
@@ -248,17 +246,16 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         for (int i = 0; i < C::LPT; ++i) *(v4i *)(stage + (wave + i * C::NW) * 1024 + lane * 16) = staged[i];
     };
 
-    // ---- block scales (fp8 only): a_scale per row of each A fragment, b_scale per 128 columns
+    // ---- block scales (fp8 only): a_scale per row of each A fragment, b_scale per 128 columns.
+    // a_scale goes through a buffer load (rows past M read as 0 instead of needing a clamp): one
+    // VGPR for the lane's row, the fragment and the K block in the scalar offset.
     constexpr int NBS = C::BLOCK_SCALE ? (C::WN + 127) / 128 : 1;
     float as_cur[C::TM], as_nxt[C::TM], bs_cur[NBS], bs_nxt[NBS];
-    uint32_t as_off[C::TM], bs_off[NBS];
+    uint32_t as_voff = 0, bs_off[NBS];
+    __amdgpu_buffer_rsrc_t ras = make_rsrc(p.as, 0);
     if constexpr (C::BLOCK_SCALE) {
-#pragma unroll
-        for (int a = 0; a < C::TM; ++a) {
-            uint32_t m = row0 + wm * C::WM + a * 16 + (lane & 15);
-            m = m < p.M ? m : p.M - 1;
-            as_off[a] = m * p.as_ms;
-        }
+        ras = make_rsrc(p.as, p.M * ((p.ksteps * C::BKB + 127) / 128) * 4);
+        as_voff = (row0 + wm * C::WM + (lane & 15)) * p.as_ms * 4;
 #pragma unroll
         for (int j = 0; j < NBS; ++j) {
             uint32_t nb = (col0 + wn * C::WN) / 128 + j;
@@ -270,7 +267,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         if constexpr (C::BLOCK_SCALE) {
             const uint32_t kb = kbeg + kt;
 #pragma unroll
-            for (int a = 0; a < C::TM; ++a) as_v[a] = p.as[as_off[a] + kb * p.as_ks];
+            for (int a = 0; a < C::TM; ++a)
+                as_v[a] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (a * 16 * p.as_ms + kb * p.as_ks) * 4, 0));
 #pragma unroll
             for (int j = 0; j < NBS; ++j) bs_v[j] = p.bs[bs_off[j] + kb * p.bs_ks];
         }
@@ -322,13 +321,13 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         // instruction i < LPT_A of this wave belongs to A, the rest to B (RBA*2 % NW == 0)
         auto issue_a1 = [&](int i, int kt, int buf) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                ra, (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024), 16, voff[i],
-                (uint32_t)kt * C::BKB, 0, 0);
+                ra, (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024), 16, voff_a,
+                load_soff(i, kt), 0, 0);
         };
         auto issue_b1 = [&](int i, int kt) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 rb, (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (wave + i * C::NW) * 1024 - C::A_BYTES), 16,
-                voff[i], (uint32_t)kt * C::BKB, 0, 0);
+                voff_b, load_soff(i, kt), 0, 0);
         };
         auto next_buf = [&](int bufi) { return bufi + 1 == NA_BUF ? 0 : bufi + 1; };
         // The copies of one slot as a numbered list 0 .. n-1, so a phase can issue them one by one.
@@ -415,7 +414,45 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 if constexpr (LATE) issue_even(j, kt_slot, GUARD);
                 else issue_odd(j, kt_slot, GUARD);
             }
+            // block scales: one factor per A-fragment row block and 128-column block for this K step
+            float sc[C::BLOCK_SCALE ? C::TM : 1][NBS];
+            if constexpr (C::BLOCK_SCALE) {
+#pragma unroll
+                for (int a = 0; a < C::TM; ++a)
+#pragma unroll
+                    for (int j = 0; j < NBS; ++j) sc[a][j] = as_cur[a] * bs_cur[j];
+            }
             auto mfma_cols = [&](int b0, int b1, int ncopy) {
+                if constexpr (C::BLOCK_SCALE) {
+                    // partial product of this 128-wide K block into a fresh accumulator, folded into
+                    // the running sum with one FMA per element (hip_mix_gemm_kernel.cpp:231-244), one
+                    // MFMA behind so the FMAs of tile i run under the MFMA of tile i+1
+                    v4f part[2];
+#pragma unroll
+                    for (int i = b0 * C::TM; i <= b1 * C::TM; ++i) {
+                        const int a = i % C::TM, b = i / C::TM;
+                        if (i < b1 * C::TM) {
+                            if (a == 0 && b < ncopy) {
+                                if constexpr (LATE) issue_even(b, kt_slot, GUARD);
+                                else issue_odd(b, kt_slot, GUARD);
+                            }
+                            if constexpr (!(DBG & 1))
+                                part[i & 1] =
+                                    mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                        }
+                        __builtin_amdgcn_sched_barrier(0);   // MFMA i first, the FMAs of tile i-1 under it
+                        if (i > b0 * C::TM) {
+                            const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
+                            const float f = sc[pa][(pb * 16) / 128];
+                            if constexpr (!(DBG & 1)) {
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f;
+                            }
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    return;
+                }
 #pragma unroll
                 for (int b = b0; b < b1; ++b) {
                     if (b < ncopy) {              // one copy in front of each of the first columns
@@ -425,17 +462,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     }
                     if constexpr (DBG & 1) continue;
 #pragma unroll
-                    for (int a = 0; a < C::TM; ++a) {
-                        if constexpr (C::BLOCK_SCALE) {
-                            const v4f part =
-                                mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                            const float sa = as_cur[a], sb = bs_cur[(b * 16) / 128];
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) acc[a][b][r] += (part[r] * sa) * sb;
-                        } else {
-                            acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
-                        }
-                    }
+                    for (int a = 0; a < C::TM; ++a)
+                        acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
                 }
             };
             mfma_cols(0, C::TN - C::TAIL, n_c < COLS_COPY ? n_c : COLS_COPY);
