@@ -28,6 +28,15 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"f8": 5000.0, "i8": 5000.0, "bf16": 2500.0, "f16": 2500.0}
 PEAK_HBM_GBS = 8000.0
 
+# HBM-side bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a plain copy of
+# known size (`--copy-calibration`).  Measured offline (bench.py cannot run under its own
+# profiler); the summary with the commands is profiles/gemm_nt_f8_256x256_pingpong_8192.md.
+# Keyed by (kernel name, M): None where no counter run exists.
+FETCH_KIB, FETCH_FACTOR = 393440.0, 2.0     # copy of 262144 KiB reads FETCH_SIZE = 131084
+WRITE_KIB, WRITE_FACTOR = 131072.0, 1.0     # copy of 262144 KiB reads WRITE_SIZE = 262144
+MEASURED_TRAFFIC_BYTES = {("256x256_w4x2_pingpong", 8192): (FETCH_KIB * FETCH_FACTOR + WRITE_KIB * WRITE_FACTOR) * 1024.0}
+
 
 def _time_launches(fn, steps, warmup):
     """-> (wall ms per step, event ms per launch)"""
@@ -85,6 +94,9 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the headline workload")
     ap.add_argument("--cpu-rows", type=int, default=256, help="rows of C the CPU baseline computes (0 = skip)")
     ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run three plain device copies of 256 MiB (the known-size kernel the FETCH_SIZE / "
+                         "WRITE_SIZE counters are scaled against) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists).", file=sys.stderr)
@@ -94,6 +106,16 @@ def main():
     import qgemm_amd as Q
     Q.load_library()                      # fails loudly if libqgemm.so is missing: there is no fallback
     assert torch.cuda.is_available(), "bench.py needs the GPU"
+    if args.copy_calibration:
+        n = 1 << 28
+        src = torch.full((n,), 3, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"bytes_read": n, "bytes_written": n, "launches": 3}}))
+        return 0
     torch.manual_seed(42)                 # seed of the reference harness, tests/includes/test_config.h:64
     dev = "cuda:0"
     M = N = K = args.size
@@ -117,7 +139,9 @@ def main():
         "config": {"workload": f"fp8-e4m3 per-matrix-scaled GEMM M=N=K={M}, A MxK and B NxK K-contiguous, bf16 out",
                    "kernel": cfg_name},
         "roofline": {"bound": "mfma", "achieved": tflops_ev, "peak": PEAK_TFLOPS["f8"], "unit": "TFLOP/s",
-                     "frac": tflops_ev / PEAK_TFLOPS["f8"], "traffic": None,
+                     "frac": tflops_ev / PEAK_TFLOPS["f8"], "traffic": MEASURED_TRAFFIC_BYTES.get((cfg_name, M)),
+                     "traffic_unit": "bytes per launch (L2 <-> fabric, rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
+                     "algorithmic_bytes": float(M * K + N * K + 2 * M * N),
                      "kernel_ms": ev_ms, "flops_per_launch": flops},
     }
 
