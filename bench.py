@@ -92,7 +92,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the headline workload")
-    ap.add_argument("--cpu-rows", type=int, default=256, help="rows of C the CPU baseline computes (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of C the CPU baseline computes (0 = skip)")
     ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three plain device copies of 256 MiB (the known-size kernel the FETCH_SIZE / "

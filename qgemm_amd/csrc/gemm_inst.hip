@@ -23,7 +23,7 @@ static hipError_t launch_variant(const GemmArgs &a, uint32_t grid, hipStream_t s
     return hipGetLastError();
 }
 
-#define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) == PIPE_PINGPONG>
+#define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) != PIPE_SIMPLE>
 #define ROWP(NAME, BM, BN, WM_, WN_, LD, PP, AUTO)                                                    \
     {NAME, INST_ARITH, (bool)INST_BLOCK, BM, BN, CFG(BM, BN, WM_, WN_, LD, PP)::THREADS,             \
      CFG(BM, BN, WM_, WN_, LD, PP)::LDS_BYTES, LD, AUTO, &launch_variant<CFG(BM, BN, WM_, WN_, LD, PP)>}
@@ -40,8 +40,13 @@ static const Variant kTable[] = {
     ROW("256x256_w2x4_vgpr", 256, 256, 2, 4, LOAD_VGPR, false),
     ROW("128x128_w2x2_vgpr", 128, 128, 2, 2, LOAD_VGPR, false),
     ROW("32x128_w1x4_vgpr", 32, 128, 1, 4, LOAD_VGPR, false),
-    ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, true),
+    ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, (bool)INST_BLOCK),
     ROWP("256x256_w2x4_pingpong", 256, 256, 2, 4, LOAD_DMA, PIPE_PINGPONG, false),
+#if INST_BLOCK   // no block-scaled form of the solo pipeline: the row is an alias, so indices agree across families
+    ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, false),
+#else
+    ROWP("256x256_w2x2_solo", 256, 256, 2, 2, LOAD_DMA, PIPE_SOLO, true),
+#endif
 };
 
 const Variant *INST_FN(int *count) {

@@ -80,7 +80,12 @@ enum Loader : int { LOAD_DMA = 0, LOAD_VGPR = 1 };
 //                  registers, its partner reads the fragments of its next tile from LDS and
 //                  starts the next global -> LDS copy.  The matrix core of every SIMD always
 //                  has one wave feeding it; barriers fall between the phases.
-enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1 };
+//   PIPE_SOLO      4 waves = 1 per SIMD, each with a 128 x 128 wave tile (64 accumulator tiles).  A
+//                  fragments are streamed two rows of MFMAs ahead, B fragments of step k+1 replace
+//                  those of step k as they die in its last two rows, copies ride between the MFMAs:
+//                  a third fewer LDS reads per MFMA than the ping-pong pipeline and one barrier
+//                  per K step.  A triple-buffered, B double-buffered in LDS (same 160 KiB).
+enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1, PIPE_SOLO = 2 };
 
 // TAIL_ (ping-pong): number of B-fragment columns of MFMAs a wave still issues after the
 // barrier that ends its compute phase, so the hand-over to its partner is hidden.
@@ -114,9 +119,11 @@ struct GemmCfg {
     static_assert(!BLOCK_SCALE || ARITH == AR_F8, "block scales are defined for fp8 only");
     static_assert(!BLOCK_SCALE || (128 % WN == 0 || WN % 128 == 0), "wave tile must align with 128-wide scale blocks");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS is 160 KiB per CU");
-    static_assert(PIPE == PIPE_SIMPLE || (NW == 8 && LOADER == LOAD_DMA), "ping-pong needs 8 waves and the DMA loader");
-    static_assert(PIPE == PIPE_SIMPLE || (RBA * 2) % NW == 0, "ping-pong: A loads must divide evenly over the waves");
-    static_assert(PIPE == PIPE_PINGPONG || (TAIL == 0 && !A3), "TAIL and A3 belong to the ping-pong pipeline");
+    static_assert(PIPE != PIPE_PINGPONG || (NW == 8 && LOADER == LOAD_DMA), "ping-pong needs 8 waves and the DMA loader");
+    static_assert(PIPE != PIPE_SOLO || (NW == 4 && LOADER == LOAD_DMA && A3 && TM == TN && TM % 4 == 0 && !BLOCK_SCALE),
+                  "solo: 4 waves, DMA loader, square wave tiles, A triple-buffered, no block scales");
+    static_assert(PIPE == PIPE_SIMPLE || (RBA * 2) % NW == 0, "A loads must divide evenly over the waves");
+    static_assert(PIPE != PIPE_SIMPLE || (TAIL == 0 && !A3), "TAIL and A3 belong to the pipelined variants");
     static_assert(TAIL >= 0 && TAIL < TN, "TAIL counts B-fragment columns");
 };
 
@@ -168,6 +175,32 @@ __device__ inline typename AccT<ARITH>::type mma128(v4i x0, v4i x1, v4i y0, v4i 
     }
 }
 
+// The same update with the accumulator pinned in place in the accumulation registers.  With all 256 of them
+// holding accumulators (solo pipeline) the register allocator otherwise routes part of them through a
+// temporary, with copies and the wait states those need between the MFMAs.  x0/y0 and x1/y1 halves of the
+// 16-byte MFMAs are issued by the caller a row apart (`half`), so no dependent pair is back to back.
+template <int ARITH>
+__device__ inline void mma128_inplace(v4i x0, v4i x1, v4i y0, v4i y1, typename AccT<ARITH>::type &c, int half) {
+    if constexpr (ARITH == AR_F8) {
+        v8i x = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        v8i y = {y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]};
+        if (half == 0) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+    } else {
+        const v4i x = half ? x1 : x0, y = half ? y1 : y0;
+        if constexpr (ARITH == AR_I8) asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+        else if constexpr (ARITH == AR_BF16) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+        else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+    }
+}
+
+// Time stamp of the DBG & 8 builds: shader cycles (per CU, not comparable between CUs), or with DBG bit 5 the
+// constant 100 MHz counter that all CUs share.
+template <int DBG>
+__device__ inline unsigned long long dbg_stamp() {
+    if constexpr (DBG & 32) return __builtin_amdgcn_s_memrealtime();
+    else return __builtin_readcyclecounter();
+}
+
 // DBG is a measurement aid for kernel bring-up (bit 0: skip the MFMAs, bit 1: skip the
 // global loads, bit 2: skip the fragment reads); the library only instantiates DBG = 0.
 template <class C, int DBG = 0>
@@ -176,7 +209,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     typedef typename AccT<C::ARITH>::type acc_t;
     unsigned long long dbg_t0 = 0, dbg_t1 = 0, dbg_t2 = 0;
-    if constexpr (DBG & 8) dbg_t0 = __builtin_readcyclecounter();
+    if constexpr (DBG & 8) dbg_t0 = dbg_stamp<DBG>();
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -186,11 +219,15 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // ---- which tile, which K slice
     uint32_t wg = blockIdx.x, z = 0;
     if (p.nsplit > 1) {
-        z = wg % p.nsplit;
-        wg /= p.nsplit;
+        z = __builtin_amdgcn_readfirstlane(wg % p.nsplit);
+        wg = __builtin_amdgcn_readfirstlane(wg / p.nsplit);
     }
     uint32_t tm, tn;
     tile_map(wg, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    // the divisions of tile_map run on the vector ALU: bring the (uniform) result back to scalar registers so
+    // that everything derived from it (buffer descriptors, scalar offsets) stays there
+    tm = __builtin_amdgcn_readfirstlane(tm);
+    tn = __builtin_amdgcn_readfirstlane(tn);
     const uint32_t row0 = tm * C::BM, col0 = tn * C::BN;
     const uint32_t kbeg = z * p.ksteps_per_split;
     const uint32_t kend = kbeg + p.ksteps_per_split < p.ksteps ? kbeg + p.ksteps_per_split : p.ksteps;
@@ -297,9 +334,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     };
 
     // ---- K loop
-    if constexpr (DBG & 8) dbg_t1 = __builtin_readcyclecounter();
-    if constexpr (C::PIPE == PIPE_PINGPONG) {
-        // Waves 4-7 ("late" group) run one phase behind waves 0-3 ("early" group).  Phases:
+    if constexpr (DBG & 8) dbg_t1 = dbg_stamp<DBG>();
+    if constexpr (C::PIPE != PIPE_SIMPLE) {
+        // (ping-pong) Waves 4-7 ("late" group) run one phase behind waves 0-3 ("early" group).  Phases:
         //   memory : ds_read all fragments of tile kt into registers
         //   compute: MFMAs of tile kt, operands all in registers
         // so whenever one wave of a SIMD is in its compute phase its partner is in its memory
@@ -322,199 +359,317 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         constexpr int LPT_A = C::LPT_A, LPT_B = C::LPT - C::LPT_A;
         // instruction i < LPT_A of this wave belongs to A, the rest to B (RBA*2 % NW == 0)
         auto issue_a1 = [&](int i, int kt, int buf) {
+            if constexpr (DBG & 2) return;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 ra, (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024), 16, voff_a,
                 load_soff(i, kt), 0, 0);
         };
         auto issue_b1 = [&](int i, int kt) {
+            if constexpr (DBG & 2) return;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 rb, (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (wave + i * C::NW) * 1024 - C::A_BYTES), 16,
                 voff_b, load_soff(i, kt), 0, 0);
         };
         auto next_buf = [&](int bufi) { return bufi + 1 == NA_BUF ? 0 : bufi + 1; };
-        // The copies of one slot as a numbered list 0 .. n-1, so a phase can issue them one by one.
-        //   even slot 2kt  : A3 ? B(kt+1)            : A(kt+1) then B(kt+1)
-        //   odd slot 2kt+1 : A3 ? A(kt+2) -> a_wr     : nothing
-        constexpr int N_EVEN = C::A3 ? LPT_B : C::LPT, N_ODD = C::A3 ? LPT_A : 0;
-        int a_wr = C::A3 ? 2 : 1;           // buffer the next A copy of this wave goes to
-        int a_rd = 0;                       // buffer holding A of the tile being read
-        // kt: tile the early group reads in this slot; guard: check the end of K
-        auto issue_even = [&](int j, int kt, bool guard) {
-            if constexpr (DBG & 2) return;
-            if (guard && kt + 1 >= nk) return;
-            if constexpr (C::A3) issue_b1(LPT_A + j, kt + 1);
-            else if (j < LPT_A) issue_a1(j, kt + 1, a_wr);
-            else issue_b1(j, kt + 1);
-        };
-        auto issue_odd = [&](int j, int kt, bool guard) {
-            if constexpr (DBG & 2) return;
-            if constexpr (C::A3) {
-                if (guard && kt + 2 >= nk) return;
-                issue_a1(j, kt + 2, a_wr);
-            }
-        };
-        v4i fa[C::TM][2], fb[C::TN][2];
-        constexpr int COLS_COPY = C::TN - C::TAIL;    // copies that can ride between the MFMA columns
-
-        // DBG bit 4: accumulate cycles per phase section (s_memtime, so only taken at points
-        // where no LDS read is outstanding)
-        unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, tprev = 0;
-        auto stamp = [&](int slot) {
-            if constexpr (DBG & 16) {
-                const unsigned long long t = __builtin_readcyclecounter();
-                ph[slot] += t - tprev;
-                tprev = t;
-            }
-        };
-
-        // one K step of one wave.  LATE / GUARD are std::integral_constant<bool>.
-        auto step = [&](int kt, auto late_tag, auto guard_tag) {
-            constexpr bool LATE = decltype(late_tag)::value, GUARD = decltype(guard_tag)::value;
-            // ---- memory phase (early: slot 2kt, even; late: slot 2kt+1, odd)
-            if constexpr (C::BLOCK_SCALE) load_scales(kt, as_cur, bs_cur);
-            const char *sa_ = smem + a_rd * C::A_BYTES;
-            const char *sb_ = smem + B_BASE + (kt & 1) * C::B_BYTES - C::A_BYTES;   // frag_b adds RBA row blocks
-            constexpr int n_m = LATE ? N_ODD : N_EVEN;     // copies of this wave in this phase
-            if (!(DBG & 4) || kt == 0) {
-#pragma unroll
-                for (int a = 0; a < C::TM; ++a) {
-                    if (a < n_m) {
-                        if constexpr (LATE) issue_odd(a, kt, GUARD);
-                        else issue_even(a, kt, GUARD);
-                    }
-                    fa[a][0] = frag_a(sa_, a, 0);
-                    fa[a][1] = frag_a(sa_, a, 1);
-                }
-#pragma unroll
-                for (int b = 0; b < C::TN; ++b) {
-                    if (C::TM + b < n_m) {
-                        if constexpr (LATE) issue_odd(C::TM + b, kt, GUARD);
-                        else issue_even(C::TM + b, kt, GUARD);
-                    }
-                    fb[b][0] = frag_b(sb_, b, 0);
-                    fb[b][1] = frag_b(sb_, b, 1);
-                }
-            }
-            if constexpr (LATE ? (N_ODD > 0) : !C::A3) a_wr = next_buf(a_wr);
-            a_rd = next_buf(a_rd);
-            __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());   // reads done before the buffers may be refilled
-            stamp(0);
-            auto wait_copies = [&]() {   // end of an odd slot: all copies landed but (A3) the A copy just issued
-                __builtin_amdgcn_sched_barrier(0);   // stays behind the MFMAs of the phase
-                if (C::A3 && (!GUARD || kt + 2 < nk)) __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
-                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        if constexpr (C::PIPE == PIPE_SOLO) {
+            // K step kt of a wave (TM rows of TN MFMAs; all B fragments and up to four A fragments in registers):
+            //   row a = 0 .. TM-1:   [copies]  read A(kt)[a+2] (last two rows: A(kt+1)[0], [1]);
+            //                        TN MFMAs  acc[a][*] += B(kt)[*] x A(kt)[a]
+            //   in the last row B(kt)[b] is dead after its MFMA and B(kt+1)[b] is read into its registers.
+            // One barrier per step, in front of row TM-2, preceded by the wait for this wave's reads and for all
+            // its copies but the A copies of this step.  Copies: A(kt+2) -> A buffer (kt+2) % 3 in rows 0 .. 3,
+            // B(kt+2) -> B buffer kt & 1 in the two rows behind the barrier.  So A(kt+1) and B(kt+1), issued a whole
+            // step earlier, are known to have landed exactly where they are first read (rows TM-2 .. TM-1), and the
+            // buffers being overwritten (A(kt-1): read before the barrier of step kt-1; B(kt): read in the last row
+            // of step kt-1, before this step's barrier) are free.  64 KiB per step at 64 B/clk per CU keeps the
+            // load path busy for half of a step: every copy gets a full step to land.
+            constexpr int TMs = C::TM;
+            constexpr int COPY_ROWS_A = 4, CPR_A = (LPT_A + COPY_ROWS_A - 1) / COPY_ROWS_A;   // A copies per row
+            constexpr int CPR_B = (LPT_B + 1) / 2;                                          // B copies per row
+            static_assert(TMs >= COPY_ROWS_A + 2, "A copies ride in front of the barrier");
+            v4i fbr[C::TN][2];         // B fragments
+            v4i far[4][2];             // A fragment ring, row a in slot a % 4
+            int a_rd = 0, a_wr = 2;
+            auto rd_a = [&](int buf, int a, int slot) {
+                if constexpr (DBG & 4) return;
+                const char *sa_ = smem + buf * C::A_BYTES;
+                far[slot][0] = frag_a(sa_, a, 0);
+                far[slot][1] = frag_a(sa_, a, 1);
             };
-            if constexpr (LATE) wait_copies();
-            stamp(1);
-            phase_barrier();
-            stamp(2);
-            // ---- compute phase (early: slot 2kt+1, odd; late: slot 2kt+2, even)
-            constexpr int n_c = LATE ? N_EVEN : N_ODD;
-            const int kt_slot = LATE ? kt + 1 : kt;
-#pragma unroll
-            for (int j = COLS_COPY; j < n_c; ++j) {        // copies that do not fit between the columns
-                if constexpr (LATE) issue_even(j, kt_slot, GUARD);
-                else issue_odd(j, kt_slot, GUARD);
-            }
-            // block scales: one factor per A-fragment row block and 128-column block for this K step
-            float sc[C::BLOCK_SCALE ? C::TM : 1][NBS];
-            if constexpr (C::BLOCK_SCALE) {
-#pragma unroll
-                for (int a = 0; a < C::TM; ++a)
-#pragma unroll
-                    for (int j = 0; j < NBS; ++j) sc[a][j] = as_cur[a] * bs_cur[j];
-            }
-            auto mfma_cols = [&](int b0, int b1, int ncopy) {
-                if constexpr (C::BLOCK_SCALE) {
-                    // partial product of this 128-wide K block into a fresh accumulator, folded into
-                    // the running sum with one FMA per element (hip_mix_gemm_kernel.cpp:231-244), one
-                    // MFMA behind so the FMAs of tile i run under the MFMA of tile i+1
-                    v4f part[2];
-#pragma unroll
-                    for (int i = b0 * C::TM; i <= b1 * C::TM; ++i) {
-                        const int a = i % C::TM, b = i / C::TM;
-                        if (i < b1 * C::TM) {
-                            if (a == 0 && b < ncopy) {
-                                if constexpr (LATE) issue_even(b, kt_slot, GUARD);
-                                else issue_odd(b, kt_slot, GUARD);
-                            }
-                            if constexpr (!(DBG & 1))
-                                part[i & 1] =
-                                    mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                        }
-                        __builtin_amdgcn_sched_barrier(0);   // MFMA i first, the FMAs of tile i-1 under it
-                        if (i > b0 * C::TM) {
-                            const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
-                            const float f = sc[pa][(pb * 16) / 128];
-                            if constexpr (!(DBG & 1)) {
-#pragma unroll
-                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f;
-                            }
-                        }
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    return;
-                }
-#pragma unroll
-                for (int b = b0; b < b1; ++b) {
-                    if (b < ncopy) {              // one copy in front of each of the first columns
-                        if constexpr (LATE) issue_even(b, kt_slot, GUARD);
-                        else issue_odd(b, kt_slot, GUARD);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    if constexpr (DBG & 1) continue;
-#pragma unroll
-                    for (int a = 0; a < C::TM; ++a)
-                        acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
-                }
+            auto rd_b = [&](int kt, int b) {
+                if constexpr (DBG & 4) return;
+                const char *sb_ = smem + B_BASE + (kt & 1) * C::B_BYTES - C::A_BYTES;   // frag_b adds RBA row blocks
+                fbr[b][0] = frag_b(sb_, b, 0);
+                fbr[b][1] = frag_b(sb_, b, 1);
             };
-            mfma_cols(0, C::TN - C::TAIL, n_c < COLS_COPY ? n_c : COLS_COPY);
-            if constexpr (LATE ? !C::A3 : (N_ODD > 0)) a_wr = next_buf(a_wr);
-            stamp(3);
-            if constexpr (!LATE) wait_copies();
-            stamp(4);
-            if (!LATE || !GUARD || kt + 1 < nk) phase_barrier();
-            stamp(5);
-            mfma_cols(C::TN - C::TAIL, C::TN, 0);
-        };
-
-        if (nk > 0) {
+            constexpr int HALVES = C::ARITH == AR_F8 ? 1 : 2;
+            auto mma = [&](int a, int b, int half) {
+                if constexpr (!(DBG & 1))
+                    mma128_inplace<C::ARITH>(fbr[b][0], fbr[b][1], far[a % 4][0], far[a % 4][1], acc[a][b], half);
+            };
+            auto step = [&](int kt, auto guard_tag) {
+                constexpr bool GUARD = decltype(guard_tag)::value;
+                const int a_nx = next_buf(a_rd);
+                const bool copies = !GUARD || kt + 2 < nk;
 #pragma unroll
-            for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
+                for (int a = 0; a < TMs; ++a) {
+                    if (a == TMs - 2 && !(DBG & 64)) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        // lgkmcnt(0) and vmcnt(LPT_A) (vmcnt(0) when this step issued no copies)
+                        if (copies) __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A) & 0xF0FF);
+                        else __builtin_amdgcn_s_waitcnt(0x0070);
+                        phase_barrier();
+                    }
+                    // the side instructions of a row go between its MFMAs, one at a time: a run of them in front
+                    // of the row would leave the matrix core idle once they take longer than one MFMA
+                    auto side = [&](int slot) {      // slot 0 .. TN-1: what rides behind MFMA `slot` of this row
+                        if (slot < 2) {              // the two halves of the A fragment two rows ahead
+                            if constexpr (DBG & 4) return;
+                            const int buf = a + 2 < TMs ? a_rd : a_nx, ar = a + 2 < TMs ? a + 2 : a + 2 - TMs;
+                            far[(a + 2) % 4][slot] = frag_a(smem + buf * C::A_BYTES, ar, slot);
+                            return;
+                        }
+                        const int j = slot - 2;      // copy j of this row
+                        if (!copies) return;
+                        if (a < COPY_ROWS_A) {
+                            if (j < CPR_A && a * CPR_A + j < LPT_A) issue_a1(a * CPR_A + j, kt + 2, a_wr);
+                        } else if (a >= TMs - 2) {
+                            const int r = a - (TMs - 2);
+                            if (j < CPR_B && r * CPR_B + j < LPT_B) issue_b1(LPT_A + r * CPR_B + j, kt + 2);
+                        }
+                    };
+                    static_assert(CPR_A + 2 <= C::TN && CPR_B + 2 <= C::TN, "side instructions of a row exceed its MFMAs");
 #pragma unroll
-            for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 0);
-            if (C::A3 && nk > 1) {
+                    for (int h = 0; h < HALVES; ++h) {
 #pragma unroll
-                for (int i = 0; i < LPT_A; ++i) issue_a1(i, 1, 1);
-                __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
-            } else {
+                        for (int b = 0; b < C::TN; ++b) {
+                            mma(a, b, h);
+                            if (h == 0) side(b);
+                            // B(kt)[b] is dead: its registers take B(kt+1)[b]
+                            if (a == TMs - 1 && h == HALVES - 1) rd_b(kt + 1, b);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                a_rd = a_nx;
+                a_wr = next_buf(a_wr);
+            };
+            typedef std::integral_constant<bool, true> yes_t;
+            typedef std::integral_constant<bool, false> no_t;
+            if (nk > 0) {
+#pragma unroll
+                for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
+#pragma unroll
+                for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 0);
+                if (nk > 1) {
+#pragma unroll
+                    for (int i = 0; i < LPT_A; ++i) issue_a1(i, 1, 1);
+#pragma unroll
+                    for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 1);
+                }
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-            }
-            phase_barrier();
-        }
-        typedef std::integral_constant<bool, true> yes_t;
-        typedef std::integral_constant<bool, false> no_t;
-        const int nk_fast = nk > 3 ? nk - 3 : 0;    // steps that cannot touch the end of K
-        if (wave >= C::NW / 2) {
-            if (nk > 0) {                   // slot 0 of the late group: only its copies
+                phase_barrier();
 #pragma unroll
-                for (int j = 0; j < N_EVEN; ++j) issue_even(j, 0, true);
-                if (!C::A3) a_wr = next_buf(a_wr);
+                for (int b = 0; b < C::TN; ++b) rd_b(0, b);
+                rd_a(0, 0, 0);
+                rd_a(0, 1, 1);
+                // B(0) is in registers everywhere before step 0 starts to overwrite its buffer
+                __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());
+                phase_barrier();
+                int kt = 0;
+                for (; kt + 2 < nk; ++kt) step(kt, no_t{});
+                for (; kt < nk; ++kt) step(kt, yes_t{});
+                __builtin_amdgcn_s_waitcnt(0x0070);      // reads of the last row done before LDS serves the epilogue
+                phase_barrier();
+                // the MFMAs above are opaque to the compiler's hazard handling: give the last one its wait states
+                // before the epilogue reads the accumulators
+                asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+            }
+        } else {
+            // The copies of one slot as a numbered list 0 .. n-1, so a phase can issue them one by one.
+            //   even slot 2kt  : A3 ? B(kt+1)            : A(kt+1) then B(kt+1)
+            //   odd slot 2kt+1 : A3 ? A(kt+2) -> a_wr     : nothing
+            constexpr int N_EVEN = C::A3 ? LPT_B : C::LPT, N_ODD = C::A3 ? LPT_A : 0;
+            int a_wr = C::A3 ? 2 : 1;           // buffer the next A copy of this wave goes to
+            int a_rd = 0;                       // buffer holding A of the tile being read
+            // kt: tile the early group reads in this slot; guard: check the end of K
+            auto issue_even = [&](int j, int kt, bool guard) {
+                if constexpr (DBG & 2) return;
+                if (guard && kt + 1 >= nk) return;
+                if constexpr (C::A3) issue_b1(LPT_A + j, kt + 1);
+                else if (j < LPT_A) issue_a1(j, kt + 1, a_wr);
+                else issue_b1(j, kt + 1);
+            };
+            auto issue_odd = [&](int j, int kt, bool guard) {
+                if constexpr (DBG & 2) return;
+                if constexpr (C::A3) {
+                    if (guard && kt + 2 >= nk) return;
+                    issue_a1(j, kt + 2, a_wr);
+                }
+            };
+            v4i fa[C::TM][2], fb[C::TN][2];
+            constexpr int COLS_COPY = C::TN - C::TAIL;    // copies that can ride between the MFMA columns
+
+            // DBG bit 4: accumulate cycles per phase section (s_memtime, so only taken at points
+            // where no LDS read is outstanding)
+            unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, tprev = 0;
+            auto stamp = [&](int slot) {
+                if constexpr (DBG & 16) {
+                    const unsigned long long t = __builtin_readcyclecounter();
+                    ph[slot] += t - tprev;
+                    tprev = t;
+                }
+            };
+
+            // one K step of one wave.  LATE / GUARD are std::integral_constant<bool>.
+            auto step = [&](int kt, auto late_tag, auto guard_tag) {
+                constexpr bool LATE = decltype(late_tag)::value, GUARD = decltype(guard_tag)::value;
+                // ---- memory phase (early: slot 2kt, even; late: slot 2kt+1, odd)
+                if constexpr (C::BLOCK_SCALE) load_scales(kt, as_cur, bs_cur);
+                const char *sa_ = smem + a_rd * C::A_BYTES;
+                const char *sb_ = smem + B_BASE + (kt & 1) * C::B_BYTES - C::A_BYTES;   // frag_b adds RBA row blocks
+                constexpr int n_m = LATE ? N_ODD : N_EVEN;     // copies of this wave in this phase
+                if (!(DBG & 4) || kt == 0) {
+    #pragma unroll
+                    for (int a = 0; a < C::TM; ++a) {
+                        if (a < n_m) {
+                            if constexpr (LATE) issue_odd(a, kt, GUARD);
+                            else issue_even(a, kt, GUARD);
+                        }
+                        fa[a][0] = frag_a(sa_, a, 0);
+                        fa[a][1] = frag_a(sa_, a, 1);
+                    }
+    #pragma unroll
+                    for (int b = 0; b < C::TN; ++b) {
+                        if (C::TM + b < n_m) {
+                            if constexpr (LATE) issue_odd(C::TM + b, kt, GUARD);
+                            else issue_even(C::TM + b, kt, GUARD);
+                        }
+                        fb[b][0] = frag_b(sb_, b, 0);
+                        fb[b][1] = frag_b(sb_, b, 1);
+                    }
+                }
+                if constexpr (LATE ? (N_ODD > 0) : !C::A3) a_wr = next_buf(a_wr);
+                a_rd = next_buf(a_rd);
+                __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());   // reads done before the buffers may be refilled
+                stamp(0);
+                auto wait_copies = [&]() {   // end of an odd slot: all copies landed but (A3) the A copy just issued
+                    __builtin_amdgcn_sched_barrier(0);   // stays behind the MFMAs of the phase
+                    if (C::A3 && (!GUARD || kt + 2 < nk)) __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
+                    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                };
+                if constexpr (LATE) wait_copies();
+                stamp(1);
+                phase_barrier();
+                stamp(2);
+                // ---- compute phase (early: slot 2kt+1, odd; late: slot 2kt+2, even)
+                constexpr int n_c = LATE ? N_EVEN : N_ODD;
+                const int kt_slot = LATE ? kt + 1 : kt;
+    #pragma unroll
+                for (int j = COLS_COPY; j < n_c; ++j) {        // copies that do not fit between the columns
+                    if constexpr (LATE) issue_even(j, kt_slot, GUARD);
+                    else issue_odd(j, kt_slot, GUARD);
+                }
+                // block scales: one factor per A-fragment row block and 128-column block for this K step
+                float sc[C::BLOCK_SCALE ? C::TM : 1][NBS];
+                if constexpr (C::BLOCK_SCALE) {
+    #pragma unroll
+                    for (int a = 0; a < C::TM; ++a)
+    #pragma unroll
+                        for (int j = 0; j < NBS; ++j) sc[a][j] = as_cur[a] * bs_cur[j];
+                }
+                auto mfma_cols = [&](int b0, int b1, int ncopy) {
+                    if constexpr (C::BLOCK_SCALE) {
+                        // partial product of this 128-wide K block into a fresh accumulator, folded into
+                        // the running sum with one FMA per element (hip_mix_gemm_kernel.cpp:231-244), one
+                        // MFMA behind so the FMAs of tile i run under the MFMA of tile i+1
+                        v4f part[2];
+    #pragma unroll
+                        for (int i = b0 * C::TM; i <= b1 * C::TM; ++i) {
+                            const int a = i % C::TM, b = i / C::TM;
+                            if (i < b1 * C::TM) {
+                                if (a == 0 && b < ncopy) {
+                                    if constexpr (LATE) issue_even(b, kt_slot, GUARD);
+                                    else issue_odd(b, kt_slot, GUARD);
+                                }
+                                if constexpr (!(DBG & 1))
+                                    part[i & 1] =
+                                        mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                            }
+                            __builtin_amdgcn_sched_barrier(0);   // MFMA i first, the FMAs of tile i-1 under it
+                            if (i > b0 * C::TM) {
+                                const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
+                                const float f = sc[pa][(pb * 16) / 128];
+                                if constexpr (!(DBG & 1)) {
+    #pragma unroll
+                                    for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f;
+                                }
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        return;
+                    }
+    #pragma unroll
+                    for (int b = b0; b < b1; ++b) {
+                        if (b < ncopy) {              // one copy in front of each of the first columns
+                            if constexpr (LATE) issue_even(b, kt_slot, GUARD);
+                            else issue_odd(b, kt_slot, GUARD);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        if constexpr (DBG & 1) continue;
+    #pragma unroll
+                        for (int a = 0; a < C::TM; ++a)
+                            acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                    }
+                };
+                mfma_cols(0, C::TN - C::TAIL, n_c < COLS_COPY ? n_c : COLS_COPY);
+                if constexpr (LATE ? !C::A3 : (N_ODD > 0)) a_wr = next_buf(a_wr);
+                stamp(3);
+                if constexpr (!LATE) wait_copies();
+                stamp(4);
+                if (!LATE || !GUARD || kt + 1 < nk) phase_barrier();
+                stamp(5);
+                mfma_cols(C::TN - C::TAIL, C::TN, 0);
+            };
+
+            if (nk > 0) {
+    #pragma unroll
+                for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
+    #pragma unroll
+                for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 0);
+                if (C::A3 && nk > 1) {
+    #pragma unroll
+                    for (int i = 0; i < LPT_A; ++i) issue_a1(i, 1, 1);
+                    __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
+                } else {
+                    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                }
                 phase_barrier();
             }
-            if constexpr (DBG & 16) tprev = __builtin_readcyclecounter();
-            int kt = 0;
-            for (; kt < nk_fast; ++kt) step(kt, yes_t{}, no_t{});
-            for (; kt < nk; ++kt) step(kt, yes_t{}, yes_t{});
-        } else {
-            if constexpr (DBG & 16) tprev = __builtin_readcyclecounter();
-            int kt = 0;
-            for (; kt < nk_fast; ++kt) step(kt, no_t{}, no_t{});
-            for (; kt < nk; ++kt) step(kt, no_t{}, yes_t{});
-        }
-        if constexpr (DBG & 16) {
-            if (lane == 0)
-                for (int i = 0; i < 6; ++i) p.dbg_cycles[((size_t)blockIdx.x * C::NW + wave) * 8 + i] = ph[i];
+            typedef std::integral_constant<bool, true> yes_t;
+            typedef std::integral_constant<bool, false> no_t;
+            const int nk_fast = nk > 3 ? nk - 3 : 0;    // steps that cannot touch the end of K
+            if (wave >= C::NW / 2) {
+                if (nk > 0) {                   // slot 0 of the late group: only its copies
+    #pragma unroll
+                    for (int j = 0; j < N_EVEN; ++j) issue_even(j, 0, true);
+                    if (!C::A3) a_wr = next_buf(a_wr);
+                    phase_barrier();
+                }
+                if constexpr (DBG & 16) tprev = __builtin_readcyclecounter();
+                int kt = 0;
+                for (; kt < nk_fast; ++kt) step(kt, yes_t{}, no_t{});
+                for (; kt < nk; ++kt) step(kt, yes_t{}, yes_t{});
+            } else {
+                if constexpr (DBG & 16) tprev = __builtin_readcyclecounter();
+                int kt = 0;
+                for (; kt < nk_fast; ++kt) step(kt, no_t{}, no_t{});
+                for (; kt < nk; ++kt) step(kt, no_t{}, yes_t{});
+            }
+            if constexpr (DBG & 16) {
+                if (lane == 0)
+                    for (int i = 0; i < 6; ++i) p.dbg_cycles[((size_t)blockIdx.x * C::NW + wave) * 8 + i] = ph[i];
+            }
         }
     } else {
         if (nk > 0) {
@@ -572,7 +727,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     }
 
-    if constexpr (DBG & 8) dbg_t2 = __builtin_readcyclecounter();
+    if constexpr (DBG & 8) dbg_t2 = dbg_stamp<DBG>();
     // ---- epilogue: lane holds C[m][n0 .. n0+3] of every 16x16 tile
     float scale = 1.0f;
     if (p.per_matrix_scale) scale = p.as[0] * p.bs[0];
@@ -581,52 +736,72 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // Fast path: the wave tile lies inside C and rows of C are 16-byte aligned.  The accumulator
     // layout (adjacent lanes = adjacent rows of C) would make every lane of a store its own
     // request; so each 16-row slab goes through this wave's private LDS scratch and leaves as
-    // whole 16-byte-per-lane rows.  LDS is free here: in the ping-pong pipeline every wave is
-    // past the barrier that follows the last fragment read of both groups; the simple pipeline
-    // needs one more barrier.
-    constexpr int EPI_PITCH = C::WN * 4 + 16;
-    constexpr int EPI_BYTES = 16 * EPI_PITCH;
-    constexpr bool EPI_FITS = C::NW * EPI_BYTES <= C::LDS_BYTES;
+    // whole 16-byte-per-lane row pieces.  Two scratch slabs per wave: slab a+1 is converted and
+    // written while slab a is read back and stored.  The output type is dispatched once, outside
+    // the slab loop, so the loop is straight-line code.  LDS is free here: the pipelined variants
+    // end their K loop with every wave past a barrier that follows the last fragment read; the
+    // simple pipeline needs one more barrier.
+    constexpr int EPI_BYTES = 16 * (C::WN * 4 + 64);
+    constexpr bool EPI_FITS = C::NW * 2 * EPI_BYTES <= C::LDS_BYTES && 64 % (C::WN * 2 / 16) == 0 && C::WN <= 256;
     if constexpr (C::PIPE == PIPE_SIMPLE && EPI_FITS) __syncthreads();
     const bool wave_tile_full = row0 + wm * C::WM + C::WM <= p.M && col0 + wn * C::WN + C::WN <= p.N;
     if (EPI_FITS && p.vec_store == 2 && wave_tile_full) {
-        char *scratch = smem + wave * EPI_BYTES;
-        const int es = dtype_bytes(p.out_dtype);
-        const int lanes_per_row = C::WN * es / 16, rows_per_pass = 64 / lanes_per_row;
-        const int rd_row = lane / lanes_per_row, rd_col = (lane % lanes_per_row) * 16;
-        char *wr = scratch + (lane & 15) * EPI_PITCH + (lane >> 4) * 4 * es;
-        const size_t c_row_bytes = (size_t)p.ldc * es;
-        char *cbase = Cz + ((size_t)(row0 + wm * C::WM) * p.ldc + col0 + wn * C::WN) * es + rd_col;
+        auto run = [&](auto dt_tag) {
+            constexpr int DT = decltype(dt_tag)::value;
+            constexpr int ES = (DT == QGEMM_DT_BF16 || DT == QGEMM_DT_F16) ? 2 : 4;
+            // row pitch: 32 bytes (2-byte outputs, 8-byte writes) or 64 bytes (4-byte outputs, 16-byte
+            // writes) past a multiple of 256, so the 16 rows a write instruction touches spread over all banks
+            constexpr int PITCH = C::WN * ES + (ES == 2 ? 32 : 64);
+            constexpr int LPR = C::WN * ES / 16;          // lanes per row when reading back
+            constexpr int RPP = 64 / LPR;                 // rows per read instruction
+            constexpr int PASSES = 16 / RPP;
+            static_assert(16 * PITCH <= EPI_BYTES && PASSES >= 1, "scratch slab");
+            char *scratch = smem + wave * (2 * EPI_BYTES);
+            const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
+            const int wr_off = (lane & 15) * PITCH + (lane >> 4) * 4 * ES;
+            const size_t c_row_bytes = (size_t)p.ldc * ES;
+            char *cbase = Cz + ((size_t)(row0 + wm * C::WM) * p.ldc + col0 + wn * C::WN) * ES + rd_col;
+            auto write_slab = [&](int a) {
+                char *wr = scratch + (a & 1) * EPI_BYTES + wr_off;
 #pragma unroll
-        for (int a = 0; a < C::TM; ++a) {
-#pragma unroll
-            for (int b = 0; b < C::TN; ++b) {
-                if (es == 4) {
-                    if (p.out_dtype == QGEMM_DT_I32) {
+                for (int b = 0; b < C::TN; ++b) {
+                    if constexpr (DT == QGEMM_DT_I32) {
                         *(acc_t *)(wr + b * 16 * 4) = acc[a][b];
-                    } else {
+                    } else if constexpr (DT == QGEMM_DT_F32) {
                         v4f v;
 #pragma unroll
                         for (int r = 0; r < 4; ++r) v[r] = (float)acc[a][b][r] * scale;
                         *(v4f *)(wr + b * 16 * 4) = v;
-                    }
-                } else {
-                    us4 h;
+                    } else {
+                        us4 h;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float v = (float)acc[a][b][r] * scale;
-                        h[r] = p.out_dtype == QGEMM_DT_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+                        for (int r = 0; r < 4; ++r) {
+                            const float v = (float)acc[a][b][r] * scale;
+                            h[r] = DT == QGEMM_DT_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+                        }
+                        *(us4 *)(wr + b * 16 * 2) = h;
                     }
-                    *(us4 *)(wr + b * 16 * 2) = h;
                 }
+            };
+            write_slab(0);
+#pragma unroll
+            for (int a = 0; a < C::TM; ++a) {
+                if (a + 1 < C::TM) write_slab(a + 1);
+                const char *rd = scratch + (a & 1) * EPI_BYTES + rd_row * PITCH + rd_col;
+                v4i v[PASSES];
+#pragma unroll
+                for (int ps = 0; ps < PASSES; ++ps) v[ps] = *(const v4i *)(rd + ps * RPP * PITCH);
+#pragma unroll
+                for (int ps = 0; ps < PASSES; ++ps)
+                    *(v4i *)(cbase + (size_t)(a * 16 + rd_row + ps * RPP) * c_row_bytes) = v[ps];
             }
-            for (int row = rd_row; row < 16; row += rows_per_pass) {
-                const v4i v = *(const v4i *)(scratch + row * EPI_PITCH + rd_col);
-                *(v4i *)(cbase + (size_t)(a * 16 + row) * c_row_bytes) = v;
-            }
-        }
+        };
+        if (p.out_dtype == QGEMM_DT_BF16) run(std::integral_constant<int, QGEMM_DT_BF16>{});
+        else if (p.out_dtype == QGEMM_DT_F16) run(std::integral_constant<int, QGEMM_DT_F16>{});
+        else if (p.out_dtype == QGEMM_DT_F32) run(std::integral_constant<int, QGEMM_DT_F32>{});
+        else run(std::integral_constant<int, QGEMM_DT_I32>{});
         if constexpr (DBG & 8) {
-            const unsigned long long t3 = __builtin_readcyclecounter();
+            const unsigned long long t3 = dbg_stamp<DBG>();
             if (lane == 0 && !(DBG & 16)) {
                 unsigned long long *o = p.dbg_cycles + ((size_t)blockIdx.x * C::NW + wave) * 4;
                 o[0] = dbg_t0; o[1] = dbg_t1; o[2] = dbg_t2; o[3] = t3;
@@ -677,7 +852,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     }
     if constexpr (DBG & 8) {
-        const unsigned long long t3 = __builtin_readcyclecounter();
+        const unsigned long long t3 = dbg_stamp<DBG>();
         if (lane == 0) {
             unsigned long long *o = p.dbg_cycles + ((size_t)blockIdx.x * C::NW + wave) * 4;
             if constexpr (!(DBG & 16)) { o[0] = dbg_t0; o[1] = dbg_t1; o[2] = dbg_t2; o[3] = t3; }

@@ -64,8 +64,12 @@ def test_golden_pattern_inputs_bf16():
 
 # ------------------------------------------------------------------ GPU half
 def _close(got, ref, what):
+    """rtol / atol of the parity bar, plus the noise floor of fp32 accumulation itself: the stored
+    results are float64 truth, and where terms of size max|ref| cancel, an fp32-accumulate result
+    (the oracle's included, see test_golden_fp8_per_matrix) is only good to ~1e-5 of that size."""
     err = np.abs(np.asarray(got, np.float64) - ref)
-    assert np.all(err <= ATOL + RTOL * np.abs(ref)), f"{what}: max err {err.max()}"
+    bound = ATOL + RTOL * np.abs(ref) + 1e-5 * np.max(np.abs(ref))
+    assert np.all(err <= bound), f"{what}: max excess {(err - bound).max()}"
 
 
 @pytest.mark.gpu
