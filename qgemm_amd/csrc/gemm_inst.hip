@@ -47,6 +47,7 @@ static const Variant kTable[] = {
 #else
     ROWP("256x256_w2x2_solo", 256, 256, 2, 2, LOAD_DMA, PIPE_SOLO, true),
 #endif
+    ROWP("256x256_w2x4_solo8", 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, false),
 };
 
 const Variant *INST_FN(int *count) {

@@ -85,6 +85,8 @@ enum Loader : int { LOAD_DMA = 0, LOAD_VGPR = 1 };
 //                  those of step k as they die in its last two rows, copies ride between the MFMAs:
 //                  a third fewer LDS reads per MFMA than the ping-pong pipeline and one barrier
 //                  per K step.  A triple-buffered, B double-buffered in LDS (same 160 KiB).
+//                  With 8 waves (128 x 64 wave tiles) the same schedule runs two waves per SIMD and
+//                  keeps the accumulators in vector registers, which the block-scale fold needs.
 enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1, PIPE_SOLO = 2 };
 
 // TAIL_ (ping-pong): number of B-fragment columns of MFMAs a wave still issues after the
@@ -120,8 +122,10 @@ struct GemmCfg {
     static_assert(!BLOCK_SCALE || (128 % WN == 0 || WN % 128 == 0), "wave tile must align with 128-wide scale blocks");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS is 160 KiB per CU");
     static_assert(PIPE != PIPE_PINGPONG || (NW == 8 && LOADER == LOAD_DMA), "ping-pong needs 8 waves and the DMA loader");
-    static_assert(PIPE != PIPE_SOLO || (NW == 4 && LOADER == LOAD_DMA && A3 && TM == TN && TM % 4 == 0 && !BLOCK_SCALE),
-                  "solo: 4 waves, DMA loader, square wave tiles, A triple-buffered, no block scales");
+    static_assert(PIPE != PIPE_SOLO || ((NW == 4 || NW == 8) && LOADER == LOAD_DMA && A3 && TM % 4 == 0 && TM >= 8 && TN >= 4),
+                  "solo: 4 or 8 waves, DMA loader, A triple-buffered, at least 8 rows of at least 4 MFMAs per step");
+    static_assert(PIPE != PIPE_SOLO || !BLOCK_SCALE || NW == 8,
+                  "solo with block scales: the accumulators have to live in the 256 vector registers of a wave");
     static_assert(PIPE == PIPE_SIMPLE || (RBA * 2) % NW == 0, "A loads must divide evenly over the waves");
     static_assert(PIPE != PIPE_SIMPLE || (TAIL == 0 && !A3), "TAIL and A3 belong to the pipelined variants");
     static_assert(TAIL >= 0 && TAIL < TN, "TAIL counts B-fragment columns");
@@ -402,15 +406,40 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 fbr[b][0] = frag_b(sb_, b, 0);
                 fbr[b][1] = frag_b(sb_, b, 1);
             };
-            constexpr int HALVES = C::ARITH == AR_F8 ? 1 : 2;
+            // 4 waves: 256 accumulator registers per lane, pinned in place (see mma128_inplace); the two
+            // halves of a 16-byte MFMA pair are then issued a row apart.  8 waves: compiler-managed.
+            constexpr bool PINNED = C::NW == 4;
+            constexpr int HALVES = (PINNED && C::ARITH != AR_F8) ? 2 : 1;
             auto mma = [&](int a, int b, int half) {
-                if constexpr (!(DBG & 1))
+                if constexpr (DBG & 1) return;
+                if constexpr (PINNED)
                     mma128_inplace<C::ARITH>(fbr[b][0], fbr[b][1], far[a % 4][0], far[a % 4][1], acc[a][b], half);
+                else
+                    acc[a][b] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % 4][0], far[a % 4][1], acc[a][b]);
             };
             auto step = [&](int kt, auto guard_tag) {
                 constexpr bool GUARD = decltype(guard_tag)::value;
                 const int a_nx = next_buf(a_rd);
                 const bool copies = !GUARD || kt + 2 < nk;
+                // block scales of this step (fetched one step ahead) and the fetch for the next one, in front of
+                // this step's copies: by the time they are used nothing older is still in flight
+                float sc[C::BLOCK_SCALE ? TMs : 1][NBS];
+                v4f part[3];
+                if constexpr (C::BLOCK_SCALE) {
+#pragma unroll
+                    for (int a = 0; a < TMs; ++a)
+#pragma unroll
+                        for (int j = 0; j < NBS; ++j) sc[a][j] = as_cur[a] * bs_cur[j];
+                    if (!GUARD || kt + 1 < nk) load_scales(kt + 1, as_cur, bs_cur);
+                }
+                auto fold = [&](int i) {
+                    if constexpr (C::BLOCK_SCALE && !(DBG & 1)) {
+                        const int pa = i / C::TN, pb = i % C::TN;
+                        const float f = sc[pa][(pb * 16) / 128];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[i % 3][r] * f;
+                    }
+                };
 #pragma unroll
                 for (int a = 0; a < TMs; ++a) {
                     if (a == TMs - 2 && !(DBG & 64)) {
@@ -439,17 +468,39 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         }
                     };
                     static_assert(CPR_A + 2 <= C::TN && CPR_B + 2 <= C::TN, "side instructions of a row exceed its MFMAs");
-#pragma unroll
-                    for (int h = 0; h < HALVES; ++h) {
+                    if constexpr (C::BLOCK_SCALE) {
+                        // each MFMA starts from zero and gives the partial product of one 128-wide K block; it is
+                        // folded into the running sum, scaled, two MFMAs later, so the four FMAs of a tile run
+                        // under the MFMAs of the next two (hip_mix_gemm_kernel.cpp:231-244)
 #pragma unroll
                         for (int b = 0; b < C::TN; ++b) {
-                            mma(a, b, h);
-                            if (h == 0) side(b);
-                            // B(kt)[b] is dead: its registers take B(kt+1)[b]
-                            if (a == TMs - 1 && h == HALVES - 1) rd_b(kt + 1, b);
+                            const int i = a * C::TN + b;
+                            if constexpr (!(DBG & 1))
+                                part[i % 3] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % 4][0], far[a % 4][1],
+                                                               v4f{0, 0, 0, 0});
+                            side(b);
+                            __builtin_amdgcn_sched_barrier(0);
+                            if (i >= 2) fold(i - 2);
+                            __builtin_amdgcn_sched_barrier(0);
+                            if (a == TMs - 1) rd_b(kt + 1, b);
+                        }
+                    } else {
+#pragma unroll
+                        for (int h = 0; h < HALVES; ++h) {
+#pragma unroll
+                            for (int b = 0; b < C::TN; ++b) {
+                                mma(a, b, h);
+                                if (h == 0) side(b);
+                                // B(kt)[b] is dead: its registers take B(kt+1)[b]
+                                if (a == TMs - 1 && h == HALVES - 1) rd_b(kt + 1, b);
+                            }
                         }
                     }
                     __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (C::BLOCK_SCALE) {
+                    fold(TMs * C::TN - 2);
+                    fold(TMs * C::TN - 1);
                 }
                 a_rd = a_nx;
                 a_wr = next_buf(a_wr);
@@ -457,6 +508,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             typedef std::integral_constant<bool, true> yes_t;
             typedef std::integral_constant<bool, false> no_t;
             if (nk > 0) {
+                if constexpr (C::BLOCK_SCALE) load_scales(0, as_cur, bs_cur);
 #pragma unroll
                 for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
 #pragma unroll
@@ -483,7 +535,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 phase_barrier();
                 // the MFMAs above are opaque to the compiler's hazard handling: give the last one its wait states
                 // before the epilogue reads the accumulators
-                asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+                if constexpr (PINNED) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
             }
         } else {
             // The copies of one slot as a numbered list 0 .. n-1, so a phase can issue them one by one.
