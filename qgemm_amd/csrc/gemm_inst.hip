@@ -40,14 +40,14 @@ static const Variant kTable[] = {
     ROW("256x256_w2x4_vgpr", 256, 256, 2, 4, LOAD_VGPR, false),
     ROW("128x128_w2x2_vgpr", 128, 128, 2, 2, LOAD_VGPR, false),
     ROW("32x128_w1x4_vgpr", 32, 128, 1, 4, LOAD_VGPR, false),
-    ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, (bool)INST_BLOCK),
+    ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, false),
     ROWP("256x256_w2x4_pingpong", 256, 256, 2, 4, LOAD_DMA, PIPE_PINGPONG, false),
 #if INST_BLOCK   // no block-scaled form of the solo pipeline: the row is an alias, so indices agree across families
     ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, false),
 #else
     ROWP("256x256_w2x2_solo", 256, 256, 2, 2, LOAD_DMA, PIPE_SOLO, true),
 #endif
-    ROWP("256x256_w2x4_solo8", 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, false),
+    ROWP("256x256_w2x4_solo8", 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, (bool)INST_BLOCK),
 };
 
 const Variant *INST_FN(int *count) {

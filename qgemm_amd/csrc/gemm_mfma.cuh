@@ -205,8 +205,10 @@ __device__ inline unsigned long long dbg_stamp() {
     else return __builtin_readcyclecounter();
 }
 
-// DBG is a measurement aid for kernel bring-up (bit 0: skip the MFMAs, bit 1: skip the
-// global loads, bit 2: skip the fragment reads); the library only instantiates DBG = 0.
+// DBG is a measurement aid for kernel bring-up; the library only instantiates DBG = 0.  Bits: 1 skip the
+// MFMAs, 2 skip the global loads, 4 skip the fragment reads, 8 per-workgroup time stamps (32: on the shared
+// 100 MHz clock), 16 per-phase cycle sums (ping-pong), 64 no barrier (solo), 128 no block-scale fold,
+// 256 constant block scales (no fetch, no cross-lane pick).  Results are wrong with any of 1 .. 4, 64 .. 256.
 template <class C, int DBG = 0>
 __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
@@ -290,15 +292,23 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     };
 
     // ---- block scales (fp8 only): a_scale per row of each A fragment, b_scale per 128 columns.
-    // a_scale goes through a buffer load (rows past M read as 0 instead of needing a clamp): one
-    // VGPR for the lane's row, the fragment and the K block in the scalar offset.
+    // a_scale is read with the rows contiguous (as_ms == 1: a_scale[m + kb*as_ks], the host guarantees it):
+    // lane l fetches the scale of wave-tile row l (and l + 64), one 256-byte request per 64 rows, through a
+    // buffer load (rows past M read as 0 or as some other finite scale; they only meet zero operands).  A
+    // step later every lane picks the row of each of its A fragments (row l & 15 of row block a) out of
+    // those registers with ds_bpermute.  One load per lane and fragment instead (16 distinct rows per
+    // instruction, every row a request of its own) keeps the texture addresser busy for longer than the
+    // MFMAs of the step take.
     constexpr int NBS = C::BLOCK_SCALE ? (C::WN + 127) / 128 : 1;
-    float as_cur[C::TM], as_nxt[C::TM], bs_cur[NBS], bs_nxt[NBS];
+    constexpr int NLD = C::BLOCK_SCALE ? (C::WM + 63) / 64 : 1;
+    float as_cur[C::TM], bs_cur[NBS], bs_raw[NBS];
+    int as_raw[NLD];
     uint32_t as_voff = 0, bs_off[NBS];
+    const int bp0 = (lane & 15) * 4;
     __amdgpu_buffer_rsrc_t ras = make_rsrc(p.as, 0);
     if constexpr (C::BLOCK_SCALE) {
         ras = make_rsrc(p.as, p.M * ((p.ksteps * C::BKB + 127) / 128) * 4);
-        as_voff = (row0 + wm * C::WM + (lane & 15)) * p.as_ms * 4;
+        as_voff = (row0 + wm * C::WM + lane) * 4;
 #pragma unroll
         for (int j = 0; j < NBS; ++j) {
             uint32_t nb = (col0 + wn * C::WN) / 128 + j;
@@ -306,15 +316,29 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             bs_off[j] = nb * p.bs_ns;
         }
     }
-    auto load_scales = [&](int kt, float *as_v, float *bs_v) {
-        if constexpr (C::BLOCK_SCALE) {
+    auto fetch_scales = [&](int kt) {          // start the loads for K step kt
+        if constexpr (C::BLOCK_SCALE && !(DBG & 256)) {
             const uint32_t kb = kbeg + kt;
 #pragma unroll
-            for (int a = 0; a < C::TM; ++a)
-                as_v[a] = __builtin_bit_cast(
-                    float, __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (a * 16 * p.as_ms + kb * p.as_ks) * 4, 0));
+            for (int j = 0; j < NLD; ++j)
+                as_raw[j] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (64 * j + kb * p.as_ks) * 4, 0);
 #pragma unroll
-            for (int j = 0; j < NBS; ++j) bs_v[j] = p.bs[bs_off[j] + kb * p.bs_ks];
+            for (int j = 0; j < NBS; ++j) bs_raw[j] = p.bs[bs_off[j] + kb * p.bs_ks];
+        }
+    };
+    auto expand_scales = [&]() {               // what fetch_scales brought becomes as_cur / bs_cur
+        if constexpr (C::BLOCK_SCALE && (DBG & 256)) {
+#pragma unroll
+            for (int a = 0; a < C::TM; ++a) as_cur[a] = 1.0f;
+#pragma unroll
+            for (int j = 0; j < NBS; ++j) bs_cur[j] = 1.0f;
+        } else if constexpr (C::BLOCK_SCALE) {
+#pragma unroll
+            for (int a = 0; a < C::TM; ++a)
+                as_cur[a] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_ds_bpermute(bp0 + ((16 * a) & 63) * 4, as_raw[(16 * a) / 64]));
+#pragma unroll
+            for (int j = 0; j < NBS; ++j) bs_cur[j] = bs_raw[j];
         }
     };
 
@@ -389,11 +413,30 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // load path busy for half of a step: every copy gets a full step to land.
             constexpr int TMs = C::TM;
             constexpr int COPY_ROWS_A = 4, CPR_A = (LPT_A + COPY_ROWS_A - 1) / COPY_ROWS_A;   // A copies per row
-            constexpr int CPR_B = (LPT_B + 1) / 2;                                          // B copies per row
-            static_assert(TMs >= COPY_ROWS_A + 2, "A copies ride in front of the barrier");
+            // A fragment ring: row a lives in slot a % RING and is read AHEAD rows before it is used (one row
+            // ahead is less than the LDS latency under load: the wave then waits in front of every row).
+            constexpr int RING = 4, AHEAD = RING / 2;
+            constexpr int BR = TMs - AHEAD;                  // row the barrier stands in front of
+            constexpr int CPR_B = (LPT_B + AHEAD - 1) / AHEAD;                              // B copies per row
+            constexpr int SLOTS = C::TN - 2;                 // MFMAs of a row a copy can ride behind
+            constexpr int CPS_A = (CPR_A + SLOTS - 1) / SLOTS, CPS_B = (CPR_B + SLOTS - 1) / SLOTS;   // copies per slot
+            static_assert(BR >= COPY_ROWS_A && TMs % RING == 0, "A copies ride in front of the barrier");
             v4i fbr[C::TN][2];         // B fragments
-            v4i far[4][2];             // A fragment ring, row a in slot a % 4
+            v4i far[RING][2];          // A fragment ring
             int a_rd = 0, a_wr = 2;
+            // block scales of the current step (as_raw / bs_raw hold what fetch_scales brought for the next)
+            int as_rc[NLD], sc_t[2] = {0, 0};
+            float bs_c[NBS], sc[2][NBS];
+            auto rotate_scales = [&]() {
+#pragma unroll
+                for (int j = 0; j < NLD; ++j) as_rc[j] = as_raw[j];
+#pragma unroll
+                for (int j = 0; j < NBS; ++j) bs_c[j] = bs_raw[j];
+            };
+            auto pick_scale = [&](const int *raw, int a) {      // a_scale of row l & 15 of row block a
+                if constexpr (DBG & 256) return __builtin_bit_cast(int, 1.0f);
+                else return __builtin_amdgcn_ds_bpermute(bp0 + ((16 * a) & 63) * 4, raw[(16 * a) / 64]);
+            };
             auto rd_a = [&](int buf, int a, int slot) {
                 if constexpr (DBG & 4) return;
                 const char *sa_ = smem + buf * C::A_BYTES;
@@ -413,9 +456,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             auto mma = [&](int a, int b, int half) {
                 if constexpr (DBG & 1) return;
                 if constexpr (PINNED)
-                    mma128_inplace<C::ARITH>(fbr[b][0], fbr[b][1], far[a % 4][0], far[a % 4][1], acc[a][b], half);
+                    mma128_inplace<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1], acc[a][b], half);
                 else
-                    acc[a][b] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % 4][0], far[a % 4][1], acc[a][b]);
+                    acc[a][b] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1], acc[a][b]);
             };
             auto step = [&](int kt, auto guard_tag) {
                 constexpr bool GUARD = decltype(guard_tag)::value;
@@ -423,26 +466,26 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 const bool copies = !GUARD || kt + 2 < nk;
                 // block scales of this step (fetched one step ahead) and the fetch for the next one, in front of
                 // this step's copies: by the time they are used nothing older is still in flight
-                float sc[C::BLOCK_SCALE ? TMs : 1][NBS];
-                v4f part[3];
+                // block scales: fetch_scales brings the a_scale rows of step kt+1 (in front of this step's
+                // copies: by the time they are used nothing older is in flight).  The factor of row a,
+                // a_scale[row] * b_scale, is made one row ahead: the cross-lane pick behind the first
+                // MFMA of row a-1, the multiply behind the second MFMA of row a, so two factors are live at a time.
+                constexpr int BEHIND = 2;      // MFMAs between a partial product and its fold
+                v4f part[BEHIND + 1];
                 if constexpr (C::BLOCK_SCALE) {
-#pragma unroll
-                    for (int a = 0; a < TMs; ++a)
-#pragma unroll
-                        for (int j = 0; j < NBS; ++j) sc[a][j] = as_cur[a] * bs_cur[j];
-                    if (!GUARD || kt + 1 < nk) load_scales(kt + 1, as_cur, bs_cur);
+                    if (!GUARD || kt + 1 < nk) fetch_scales(kt + 1);
                 }
                 auto fold = [&](int i) {
-                    if constexpr (C::BLOCK_SCALE && !(DBG & 1)) {
+                    if constexpr (C::BLOCK_SCALE && !(DBG & 1) && !(DBG & 128)) {
                         const int pa = i / C::TN, pb = i % C::TN;
-                        const float f = sc[pa][(pb * 16) / 128];
+                        const float f = sc[pa % 2][(pb * 16) / 128];
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[i % 3][r] * f;
+                        for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[i % (BEHIND + 1)][r] * f;
                     }
                 };
 #pragma unroll
                 for (int a = 0; a < TMs; ++a) {
-                    if (a == TMs - 2 && !(DBG & 64)) {
+                    if (a == BR && !(DBG & 64)) {
                         __builtin_amdgcn_sched_barrier(0);
                         // lgkmcnt(0) and vmcnt(LPT_A) (vmcnt(0) when this step issued no copies)
                         if (copies) __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A) & 0xF0FF);
@@ -452,22 +495,25 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     // the side instructions of a row go between its MFMAs, one at a time: a run of them in front
                     // of the row would leave the matrix core idle once they take longer than one MFMA
                     auto side = [&](int slot) {      // slot 0 .. TN-1: what rides behind MFMA `slot` of this row
-                        if (slot < 2) {              // the two halves of the A fragment two rows ahead
+                        if (slot < 2) {              // the two halves of the A fragment AHEAD rows ahead
                             if constexpr (DBG & 4) return;
-                            const int buf = a + 2 < TMs ? a_rd : a_nx, ar = a + 2 < TMs ? a + 2 : a + 2 - TMs;
-                            far[(a + 2) % 4][slot] = frag_a(smem + buf * C::A_BYTES, ar, slot);
+                            const int an = a + AHEAD;
+                            const int buf = an < TMs ? a_rd : a_nx, ar = an < TMs ? an : an - TMs;
+                            far[an % RING][slot] = frag_a(smem + buf * C::A_BYTES, ar, slot);
                             return;
                         }
-                        const int j = slot - 2;      // copy j of this row
                         if (!copies) return;
                         if (a < COPY_ROWS_A) {
-                            if (j < CPR_A && a * CPR_A + j < LPT_A) issue_a1(a * CPR_A + j, kt + 2, a_wr);
-                        } else if (a >= TMs - 2) {
-                            const int r = a - (TMs - 2);
-                            if (j < CPR_B && r * CPR_B + j < LPT_B) issue_b1(LPT_A + r * CPR_B + j, kt + 2);
+#pragma unroll
+                            for (int j = (slot - 2) * CPS_A; j < (slot - 1) * CPS_A; ++j)
+                                if (j < CPR_A && a * CPR_A + j < LPT_A) issue_a1(a * CPR_A + j, kt + 2, a_wr);
+                        } else if (a >= BR) {
+                            const int r = a - BR;
+#pragma unroll
+                            for (int j = (slot - 2) * CPS_B; j < (slot - 1) * CPS_B; ++j)
+                                if (j < CPR_B && r * CPR_B + j < LPT_B) issue_b1(LPT_A + r * CPR_B + j, kt + 2);
                         }
                     };
-                    static_assert(CPR_A + 2 <= C::TN && CPR_B + 2 <= C::TN, "side instructions of a row exceed its MFMAs");
                     if constexpr (C::BLOCK_SCALE) {
                         // each MFMA starts from zero and gives the partial product of one 128-wide K block; it is
                         // folded into the running sum, scaled, two MFMAs later, so the four FMAs of a tile run
@@ -476,11 +522,20 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         for (int b = 0; b < C::TN; ++b) {
                             const int i = a * C::TN + b;
                             if constexpr (!(DBG & 1))
-                                part[i % 3] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % 4][0], far[a % 4][1],
-                                                               v4f{0, 0, 0, 0});
+                                part[i % (BEHIND + 1)] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0],
+                                                               far[a % RING][1], v4f{0, 0, 0, 0});
                             side(b);
+                            if (b == 0) {        // cross-lane pick for the next row, a row's worth of MFMAs ahead
+                                if (a + 1 < TMs) sc_t[(a + 1) % 2] = pick_scale(as_rc, a + 1);
+                                else sc_t[0] = pick_scale(as_raw, 0);      // row 0 of the next step
+                            }
+                            if (b == 1) {        // factor of this row, first used behind the next MFMA
+#pragma unroll
+                                for (int j = 0; j < NBS; ++j)
+                                    sc[a % 2][j] = __builtin_bit_cast(float, sc_t[a % 2]) * bs_c[j];
+                            }
                             __builtin_amdgcn_sched_barrier(0);
-                            if (i >= 2) fold(i - 2);
+                            if (i >= BEHIND) fold(i - BEHIND);
                             __builtin_amdgcn_sched_barrier(0);
                             if (a == TMs - 1) rd_b(kt + 1, b);
                         }
@@ -499,8 +554,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if constexpr (C::BLOCK_SCALE) {
-                    fold(TMs * C::TN - 2);
-                    fold(TMs * C::TN - 1);
+#pragma unroll
+                    for (int i = TMs * C::TN - BEHIND; i < TMs * C::TN; ++i) fold(i);
+                    rotate_scales();
                 }
                 a_rd = a_nx;
                 a_wr = next_buf(a_wr);
@@ -508,7 +564,11 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             typedef std::integral_constant<bool, true> yes_t;
             typedef std::integral_constant<bool, false> no_t;
             if (nk > 0) {
-                if constexpr (C::BLOCK_SCALE) load_scales(0, as_cur, bs_cur);
+                if constexpr (C::BLOCK_SCALE) {
+                    fetch_scales(0);
+                    rotate_scales();
+                    sc_t[0] = pick_scale(as_rc, 0);
+                }
 #pragma unroll
                 for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
 #pragma unroll
@@ -523,8 +583,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 phase_barrier();
 #pragma unroll
                 for (int b = 0; b < C::TN; ++b) rd_b(0, b);
-                rd_a(0, 0, 0);
-                rd_a(0, 1, 1);
+#pragma unroll
+                for (int r = 0; r < AHEAD; ++r) rd_a(0, r, r);
                 // B(0) is in registers everywhere before step 0 starts to overwrite its buffer
                 __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());
                 phase_barrier();
@@ -577,7 +637,10 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             auto step = [&](int kt, auto late_tag, auto guard_tag) {
                 constexpr bool LATE = decltype(late_tag)::value, GUARD = decltype(guard_tag)::value;
                 // ---- memory phase (early: slot 2kt, even; late: slot 2kt+1, odd)
-                if constexpr (C::BLOCK_SCALE) load_scales(kt, as_cur, bs_cur);
+                if constexpr (C::BLOCK_SCALE) {
+                    expand_scales();
+                    if (!GUARD || kt + 1 < nk) fetch_scales(kt + 1);
+                }
                 const char *sa_ = smem + a_rd * C::A_BYTES;
                 const char *sb_ = smem + B_BASE + (kt & 1) * C::B_BYTES - C::A_BYTES;   // frag_b adds RBA row blocks
                 constexpr int n_m = LATE ? N_ODD : N_EVEN;     // copies of this wave in this phase
@@ -685,6 +748,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             };
 
             if (nk > 0) {
+                fetch_scales(0);
     #pragma unroll
                 for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
     #pragma unroll
@@ -731,22 +795,17 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 fetch_stage(0);
                 commit_stage(0);
             }
-            load_scales(0, as_nxt, bs_nxt);
+            fetch_scales(0);
         }
         for (int kt = 0; kt < nk; ++kt) {
             if constexpr (C::LOADER == LOAD_DMA)
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // this wave's part of tile kt has landed
             __syncthreads();                                 // ... and everybody else's; tile kt-1 is fully consumed
-            if constexpr (C::BLOCK_SCALE) {
-#pragma unroll
-                for (int a = 0; a < C::TM; ++a) as_cur[a] = as_nxt[a];
-#pragma unroll
-                for (int j = 0; j < NBS; ++j) bs_cur[j] = bs_nxt[j];
-            }
+            expand_scales();
             if (kt + 1 < nk) {
                 if constexpr (C::LOADER == LOAD_DMA) issue_stage(kt + 1);
                 else fetch_stage(kt + 1);
-                load_scales(kt + 1, as_nxt, bs_nxt);
+                fetch_scales(kt + 1);
             }
             const char *stage = smem + (kt & 1) * C::STAGE_BYTES;
             v4i fa[C::TM][2];

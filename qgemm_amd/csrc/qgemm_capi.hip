@@ -260,14 +260,43 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
 }
 
 // plan, get the split workspace (plus `extra` bytes behind it for transposed operands), run
-int launch_nt(const NtProblem &q, hipStream_t stream) {
+int launch_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t N, hipStream_t stream);
+
+// The MFMA kernels read a_scale with the rows contiguous (a_scale[m + kb*M], the reference's own
+// arrangement, hip_mix_gemm_kernel.cpp:149): 64 rows of one K block are one 256-byte request.  Scales
+// given with K contiguous (a_scale[m*KB + kb]) are brought to that form first: M*KB floats, a few
+// microseconds.  `room` is where in the workspace the copy goes.
+int scales_rows_contiguous(NtProblem &q, void *room, hipStream_t stream) {
+    if (!q.block || q.as_ms == 1) return QGEMM_OK;
+    const size_t KB = (q.Kbytes + 127) / 128;
+    int st = launch_transpose(4, q.as, room, q.M, KB, stream);
+    if (st != QGEMM_OK) return st;
+    q.as = (const float *)room;
+    q.as_ms = 1;
+    q.as_ks = (uint32_t)q.M;
+    return QGEMM_OK;
+}
+size_t scales_room(const NtProblem &q) {
+    if (!q.block || q.as_ms == 1) return 0;
+    return (q.M * ((q.Kbytes + 127) / 128) * 4 + 255) / 256 * 256;
+}
+
+int launch_nt(NtProblem q, hipStream_t stream) {
     Plan pl;
     int st = plan_nt(q, pl);
     if (st != QGEMM_OK) return st;
     void *ws = nullptr;
-    if (pl.split_bytes) {
-        st = ensure_workspace_locked(pl.split_bytes, &ws);
+    const size_t split_room = (pl.split_bytes + 255) / 256 * 256, as_room = scales_room(q);
+    if (split_room + as_room) {
+        st = ensure_workspace_locked(split_room + as_room, &ws);
         if (st != QGEMM_OK) return st;
+    }
+    if (as_room) {
+        st = scales_rows_contiguous(q, (char *)ws + split_room, stream);
+        if (st != QGEMM_OK) return st;
+        pl.a.as = q.as;
+        pl.a.as_ms = q.as_ms;
+        pl.a.as_ks = q.as_ks;
     }
     return run_nt(q, pl, ws, stream);
 }
