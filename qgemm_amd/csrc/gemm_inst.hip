@@ -48,6 +48,11 @@ static const Variant kTable[] = {
     ROWP("256x256_w2x2_solo", 256, 256, 2, 2, LOAD_DMA, PIPE_SOLO, true),
 #endif
     ROWP("256x256_w2x4_solo8", 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, (bool)INST_BLOCK),
+    // narrow tiles for skinny M: N / 32 workgroups stream disjoint strips of B over the whole of K, so no
+    // K split (and no second pass over partial sums) is needed to occupy the CUs
+    ROW("128x32_w4x1_dma", 128, 32, 4, 1, LOAD_DMA, true),
+    ROW("64x32_w4x1_dma", 64, 32, 4, 1, LOAD_DMA, true),
+    ROW("16x32_w1x2_dma", 16, 32, 1, 2, LOAD_DMA, true),
 };
 
 const Variant *INST_FN(int *count) {

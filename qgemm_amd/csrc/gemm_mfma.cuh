@@ -115,7 +115,14 @@ struct GemmCfg {
     static constexpr int A_BYTES = RBA * 2048, B_BYTES = RBB * 2048;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int LPT_A = RBA * 2 / NW;                  // A load instructions per wave (ping-pong)
-    static constexpr int LDS_BYTES = A3 ? 3 * A_BYTES + 2 * B_BYTES : 2 * STAGE_BYTES;
+    // simple pipeline with the DMA loader: as many stages in flight as LDS and the 6-bit vmcnt allow (at most
+    // 8).  A workgroup that streams a narrow strip of B (skinny M) otherwise waits one full memory round trip
+    // per K step.  The block-scale form keeps two (its scale loads share vmcnt with the copies).
+    static constexpr int NSTAGE_FIT = (160 * 1024) / STAGE_BYTES, NSTAGE_CNT = 2 + 63 / LPT;
+    static constexpr int NSTAGE = (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE) ? 2
+                                  : (NSTAGE_FIT < NSTAGE_CNT ? (NSTAGE_FIT < 8 ? NSTAGE_FIT : 8)
+                                                             : (NSTAGE_CNT < 8 ? NSTAGE_CNT : 8));
+    static constexpr int LDS_BYTES = A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES;
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
     static_assert(NLOAD % NW == 0, "load instructions must divide evenly over the waves");
     static_assert(!BLOCK_SCALE || ARITH == AR_F8, "block scales are defined for fp8 only");
@@ -267,7 +274,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     };
 
     auto issue_stage = [&](int kt) {       // LOAD_DMA: global -> LDS
-        char *stage = smem + (kt & 1) * C::STAGE_BYTES;
+        char *stage = smem + (kt % C::NSTAGE) * C::STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < C::LPT; ++i) {
             lds_void *dst = (lds_void *)(stage + (wave + i * C::NW) * 1024);
@@ -788,9 +795,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             }
         }
     } else {
+        constexpr int NS = C::NSTAGE;
         if (nk > 0) {
             if constexpr (C::LOADER == LOAD_DMA) {
-                issue_stage(0);
+#pragma unroll
+                for (int j = 0; j < NS - 1; ++j)
+                    if (j < nk) issue_stage(j);
             } else {
                 fetch_stage(0);
                 commit_stage(0);
@@ -798,16 +808,20 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             fetch_scales(0);
         }
         for (int kt = 0; kt < nk; ++kt) {
-            if constexpr (C::LOADER == LOAD_DMA)
-                __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // this wave's part of tile kt has landed
+            if constexpr (C::LOADER == LOAD_DMA) {
+                // this wave's part of tile kt has landed: everything but the NS-2 stages issued after it
+                // (near the end of K fewer are in flight: wait for all)
+                if (NS > 2 && kt + NS - 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * C::LPT));
+                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            }
             __syncthreads();                                 // ... and everybody else's; tile kt-1 is fully consumed
             expand_scales();
-            if (kt + 1 < nk) {
-                if constexpr (C::LOADER == LOAD_DMA) issue_stage(kt + 1);
+            if (kt + NS - 1 < nk) {                          // into the buffer tile kt-1 has just left
+                if constexpr (C::LOADER == LOAD_DMA) issue_stage(kt + NS - 1);
                 else fetch_stage(kt + 1);
-                fetch_scales(kt + 1);
             }
-            const char *stage = smem + (kt & 1) * C::STAGE_BYTES;
+            if (kt + 1 < nk) fetch_scales(kt + 1);
+            const char *stage = smem + (kt % NS) * C::STAGE_BYTES;
             v4i fa[C::TM][2];
 #pragma unroll
             for (int a = 0; a < C::TM; ++a) {
@@ -853,10 +867,10 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // end their K loop with every wave past a barrier that follows the last fragment read; the
     // simple pipeline needs one more barrier.
     constexpr int EPI_BYTES = 16 * (C::WN * 4 + 64);
-    constexpr bool EPI_FITS = C::NW * 2 * EPI_BYTES <= C::LDS_BYTES && 64 % (C::WN * 2 / 16) == 0 && C::WN <= 256;
+    constexpr bool EPI_FITS = C::NW * 2 * EPI_BYTES <= C::LDS_BYTES && C::WN >= 32 && 64 % (C::WN * 2 / 16) == 0 && C::WN <= 256;
     if constexpr (C::PIPE == PIPE_SIMPLE && EPI_FITS) __syncthreads();
     const bool wave_tile_full = row0 + wm * C::WM + C::WM <= p.M && col0 + wn * C::WN + C::WN <= p.N;
-    if (EPI_FITS && p.vec_store == 2 && wave_tile_full) {
+    if constexpr (EPI_FITS) if (p.vec_store == 2 && wave_tile_full) {
         auto run = [&](auto dt_tag) {
             constexpr int DT = decltype(dt_tag)::value;
             constexpr int ES = (DT == QGEMM_DT_BF16 || DT == QGEMM_DT_F16) ? 2 : 4;

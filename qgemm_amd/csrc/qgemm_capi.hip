@@ -141,7 +141,7 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, int cus) {
         if (!tab[i].auto_ok || (size_t)tab[i].bm > m16 || (size_t)tab[i].bm < target) continue;
         const size_t tiles = ((M + tab[i].bm - 1) / tab[i].bm) * ((N + tab[i].bn - 1) / tab[i].bn);
         const size_t area = (size_t)tab[i].bm * tab[i].bn;
-        if (tiles >= (size_t)cus && area > best_area) {
+        if (tiles * 4 >= (size_t)cus * 3 && area > best_area) {     // at least three quarters of the CUs get a tile
             best = i;
             best_area = area;
         }

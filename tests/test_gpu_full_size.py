@@ -127,7 +127,8 @@ def test_cfg4_fp8_block_scaled_6144x4608x7168():
 
 @pytest.mark.parametrize("M", [16, 64, 128])
 def test_cfg5_skinny_split_k(M):
-    """Skinny split-K, N=7168, K=2048, int8 (bit-exact) and fp8 (tolerance) with per-matrix scales; whole matrix."""
+    """Skinny M, N=7168, K=2048, int8 (bit-exact) and fp8 (tolerance) with per-matrix scales; whole matrix.
+    Once the way the heuristic runs it (narrow tiles over the whole of K) and once with K split in four."""
     N, K = 7168, 2048
     say("cfg5 skinny", M)
     qa, sa = R.quantize_int8(R.fill_normal((M, K), 42))
@@ -135,8 +136,11 @@ def test_cfg5_skinny_split_k(M):
     acc = R.gemm_i8_i32(qa, qb)
     c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
     Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), c)
-    assert "splitk" in Q.last_config(), Q.last_config()       # the heuristic splits K for this shape
-    assert np.array_equal(host(c), acc)
+    assert np.array_equal(host(c), acc), Q.last_config()
+    c.fill_(-1)
+    Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), c, split_k=4)
+    assert "splitk4" in Q.last_config(), Q.last_config()
+    assert np.array_equal(host(c), acc), Q.last_config()
     cf = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), cf)
     assert np.array_equal(host(cf), R.scale_i32_to_f32(acc, sa, sb))
@@ -144,5 +148,7 @@ def test_cfg5_skinny_split_k(M):
     fb, tb = R.quantize_fp8(R.fill_normal((N, K), 45))
     cb = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
     Q.scaled_gemm(fp8_tensor(fa), fp8_tensor(fb), scalar(ta), scalar(tb), cb, M, N, K, Q.SCALE_PER_MATRIX)
-    assert_close(host(cb), R.gemm_f32acc(R.decode_fp8(fa), R.decode_fp8(fb)) * np.float32(ta * tb),
-                 what=Q.last_config())
+    fref = R.gemm_f32acc(R.decode_fp8(fa), R.decode_fp8(fb)) * np.float32(ta * tb)
+    assert_close(host(cb), fref, what=Q.last_config())
+    Q.scaled_gemm(fp8_tensor(fa), fp8_tensor(fb), scalar(ta), scalar(tb), cb, M, N, K, Q.SCALE_PER_MATRIX, split_k=4)
+    assert_close(host(cb), fref, what=Q.last_config())
