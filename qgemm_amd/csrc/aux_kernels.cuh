@@ -126,6 +126,54 @@ __global__ void __launch_bounds__(256) transpose_kernel(const T *__restrict__ in
 }
 
 // ---------------------------------------------------------------------------
+// Byte transpose for shapes with M % 16 == 0, N % 4 == 0 and 16-byte aligned rows (the fp8 / int8
+// operands of the reference layout).  128 x 128 tile, 256 threads.  A thread loads 4 x 4 bytes (four
+// rows, one dword each: a wave reads whole 128-byte row pieces), transposes the 4 x 4 block in
+// registers with byte permutes, and writes the four resulting dwords (4 consecutive m of one n)
+// into the LDS tile [n][m]; the tile leaves as 16-byte pieces of output rows, 128 bytes per row.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) transpose_bytes_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
+                                                              uint32_t M, uint32_t N) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int T = 128, PITCH = T + 16;        // bytes per LDS row
+    __shared__ __attribute__((aligned(16))) uint8_t tile[T * PITCH];
+    const uint32_t m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+    const int cg = threadIdx.x & 31, rg = threadIdx.x >> 5;      // 32 column groups of 4 bytes x 8 row groups of 16
+    const uint32_t n = n0 + cg * 4;
+#pragma unroll
+    for (int ch = 0; ch < 4; ++ch) {
+        const uint32_t m = m0 + rg * 16 + ch * 4;
+        uint32_t a = 0, b = 0, c = 0, d = 0;
+        if (n < N && m < M) {                     // M % 4 == 0: the four rows are all inside or all outside
+            const uint8_t *src = in + (size_t)m * N + n;
+            a = *(const uint32_t *)src;
+            b = *(const uint32_t *)(src + N);
+            c = *(const uint32_t *)(src + 2 * (size_t)N);
+            d = *(const uint32_t *)(src + 3 * (size_t)N);
+        }
+        // v_perm_b32: selector byte k picks byte k of the result out of {src1 bytes 0-3, src0 bytes 4-7}
+        const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400), ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602);
+        const uint32_t cd_lo = __builtin_amdgcn_perm(d, c, 0x05010400), cd_hi = __builtin_amdgcn_perm(d, c, 0x07030602);
+        const uint32_t o0 = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100), o1 = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302);
+        const uint32_t o2 = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100), o3 = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302);
+        uint8_t *dst = tile + (cg * 4) * PITCH + rg * 16 + ch * 4;   // [n - n0][m - m0]
+        *(uint32_t *)dst = o0;
+        *(uint32_t *)(dst + PITCH) = o1;
+        *(uint32_t *)(dst + 2 * PITCH) = o2;
+        *(uint32_t *)(dst + 3 * PITCH) = o3;
+    }
+    __syncthreads();
+    const int piece = threadIdx.x & 7, row = threadIdx.x >> 3;   // 8 pieces of 16 bytes per output row, 32 rows per pass
+#pragma unroll
+    for (int ps = 0; ps < 4; ++ps) {
+        const int r = row + ps * 32;
+        const uint32_t on = n0 + r, om = m0 + piece * 16;
+        if (on < N && om < M) *(v4i *)(out + (size_t)on * M + om) = *(const v4i *)(tile + r * PITCH + piece * 16);
+    }
+#endif
+}
+
+// ---------------------------------------------------------------------------
 // Split-K second pass: C[m,n] = cast(scale * sum_z part[z][m,n]), z ascending
 // (a fixed order, so results do not depend on scheduling; int32 stays exact).
 // ---------------------------------------------------------------------------

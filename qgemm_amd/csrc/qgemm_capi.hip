@@ -324,6 +324,12 @@ int launch_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t
     if (M >= ((size_t)1 << 31) || N >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
     dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
     if (grid.y > 65535u * 1024u) return QGEMM_ERR_TOO_LARGE;
+    if (elem_bytes == 1 && M % 16 == 0 && N % 4 == 0 && (uintptr_t)in % 4 == 0 && (uintptr_t)out % 16 == 0) {
+        dim3 g128((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128));
+        hipLaunchKernelGGL(transpose_bytes_kernel, g128, dim3(256), 0, stream, (const uint8_t *)in, (uint8_t *)out,
+                           (uint32_t)M, (uint32_t)N);
+        return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
+    }
     switch (elem_bytes) {
         case 1:
             hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, dim3(256), 0, stream, (const uint8_t *)in, (uint8_t *)out,
