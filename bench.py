@@ -31,11 +31,11 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a plain copy of
 # known size (`--copy-calibration`).  Measured offline (bench.py cannot run under its own
-# profiler); the summary with the commands is profiles/gemm_nt_f8_256x256_pingpong_8192.md.
+# profiler); the summary with the commands is profiles/gemm_nt_f8_256x256_solo_8192.md.
 # Keyed by (kernel name, M): None where no counter run exists.
-FETCH_KIB, FETCH_FACTOR = 393440.0, 2.0     # copy of 262144 KiB reads FETCH_SIZE = 131084
-WRITE_KIB, WRITE_FACTOR = 131072.0, 1.0     # copy of 262144 KiB reads WRITE_SIZE = 262144
-MEASURED_TRAFFIC_BYTES = {("256x256_w4x2_pingpong", 8192): (FETCH_KIB * FETCH_FACTOR + WRITE_KIB * WRITE_FACTOR) * 1024.0}
+FETCH_KIB, FETCH_FACTOR = 405700.0, 2.0     # copy of 262144 KiB reads FETCH_SIZE = 131084
+WRITE_KIB, WRITE_FACTOR = 155648.0, 1.0     # copy of 262144 KiB reads WRITE_SIZE = 262144
+MEASURED_TRAFFIC_BYTES = {("256x256_w2x2_solo", 8192): (FETCH_KIB * FETCH_FACTOR + WRITE_KIB * WRITE_FACTOR) * 1024.0}
 
 
 def _time_launches(fn, steps, warmup):
@@ -92,7 +92,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the headline workload")
-    ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of C the CPU baseline computes (0 = skip)")
+    ap.add_argument("--cpu-rows", type=int, default=8192, help="rows of C the CPU baseline computes (0 = skip)")
     ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three plain device copies of 256 MiB (the known-size kernel the FETCH_SIZE / "
@@ -201,6 +201,23 @@ def main():
                 "tflops": 2.0 * m5 * n5 * k5 / ms / 1e9, "GBps": nbytes / ms / 1e6,
                 "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS, "ms": ms, "kernel": Q.last_config()}
             del b5s
+        # cfg 4 in the reference's own storage (A is K x M, B is K x N, scales [K/128, M] and [K/128, N/128]):
+        # two byte transposes in front of the same kernel
+        a4r, _ = _quant_fp8(torch.randn(k4, m4, device=dev))
+        b4r, _ = _quant_fp8(torch.randn(k4, n4, device=dev))
+        as4r = torch.rand(k4 // 128, m4, device=dev) * 1.5 + 0.5
+        bs4r = torch.rand(k4 // 128, n4 // 128, device=dev) * 1.5 + 0.5
+        c4r = torch.empty(m4, n4, dtype=torch.bfloat16, device=dev)
+        _, ms = _time_launches(lambda: Q.fp8_mm(a4r.t(), b4r.t(), as4r.t(), bs4r.t(), c4r), 20, 3)
+        extra["cfg4_reference_layout_fp8_mm"] = {"tflops": 2.0 * m4 * n4 * k4 / ms / 1e9, "ms": ms, "kernel": Q.last_config()}
+        del a4r, b4r, c4r
+        # transpose utility (HBM-bound: 2 * M * N * element bytes)
+        for (mt, nt, dtt, nm) in ((8192, 8192, torch.bfloat16, "2B"), (7168, 6144, torch.uint8, "1B")):
+            xt = torch.randint(0, 100, (mt, nt), device=dev).to(dtt)
+            yt = torch.empty(nt, mt, dtype=dtt, device=dev)
+            _, ms = _time_launches(lambda: Q.matrix_transpose(xt, yt), 20, 3)
+            gbs = 2.0 * mt * nt * xt.element_size() / ms / 1e6
+            extra["transpose_%s_%dx%d" % (nm, mt, nt)] = {"GBps": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS, "ms": ms}
         out["extra"] = extra
 
     # ---- CPU baseline beside it (bounded sample), and a parity spot check of the timed kernel against it
