@@ -218,6 +218,14 @@ def main():
             _, ms = _time_launches(lambda: Q.matrix_transpose(xt, yt), 20, 3)
             gbs = 2.0 * mt * nt * xt.element_size() / ms / 1e6
             extra["transpose_%s_%dx%d" % (nm, mt, nt)] = {"GBps": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS, "ms": ms}
+        # quantisers (HBM-bound): bytes = input (twice for the two-pass per-matrix form) + one output byte
+        xq = torch.randn(m4, k4, device=dev)
+        for (mode, nm, passes) in ((Q.QUANT_PER_MATRIX, "per_matrix", 2), (Q.QUANT_BLOCK_1x128, "1x128", 1),
+                                   (Q.QUANT_BLOCK_128x128, "128x128", 1)):
+            _, ms = _time_launches(lambda: Q.quantize(xq, torch.float8_e4m3fn, mode), 20, 3)
+            gbs = m4 * k4 * (4.0 * passes + 1.0) / ms / 1e6
+            extra["quantize_fp8_%s_f32_%dx%d" % (nm, m4, k4)] = {"GBps": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS, "ms": ms}
+        del xq
         out["extra"] = extra
 
     # ---- CPU baseline beside it (bounded sample), and a parity spot check of the timed kernel against it

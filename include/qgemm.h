@@ -106,6 +106,24 @@ int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, int layout, c
  * handles 2-byte elements with M % 64 == 0 and N % 32 == 0 only; any M, N here. */
 int qgemm_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t N, void *stream);
 
+/* Quantiser for the operands of qgemm_scaled_gemm: the Q_A / Q_B of C = (A o Q_A) x (B o Q_B) that
+ * README.md:1 of the reference describes ("input matrix will be quantized") and no file of it implements.
+ *   x        rows x cols, F32 / BF16 / F16, row stride ld elements (device)
+ *   q        rows x cols bytes (I8 or F8E4M3), row stride ldq
+ *   scales   QGEMM_QUANT_PER_MATRIX: 1 float, s = max|x| / 127 (int8) or / 448 (fp8)
+ *            QGEMM_QUANT_BLOCK_1x128 / _128x128 (fp8 only): one float per block, written to
+ *            scales[ib * scale_rs + jb * scale_cs] (ib: block row, jb: block column; strides in floats),
+ *            so the a_scale / b_scale arrangement of either layout of qgemm_scaled_gemm can be produced
+ *            directly (hip_mix_gemm_kernel.cpp:137,149)
+ * q = round-to-nearest-even(x / s), saturated to +-127 / +-448; an all-zero block gets s = 1. */
+typedef enum qgemm_quant_mode {
+    QGEMM_QUANT_PER_MATRIX = 1,
+    QGEMM_QUANT_BLOCK_1x128 = 2,
+    QGEMM_QUANT_BLOCK_128x128 = 3
+} qgemm_quant_mode_t;
+int qgemm_quantize(int in_dtype, int out_dtype, int mode, const void *x, size_t ld, size_t rows, size_t cols, void *q,
+                   size_t ldq, float *scales, size_t scale_rs, size_t scale_cs, void *stream);
+
 /* Tile raster used by the GEMM kernels: linear workgroup id -> (tile_m, tile_n).
  * Replaces the GROUP_SIZE_M swizzle of src/gemm/sm89_gemm_kernel_v3.cu:169-183
  * (and fixes its clamp), composed with the 8-XCD remap the reference only names

@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "aux_kernels.cuh"
+#include "quant_kernels.cuh"
 #include "selftest.cuh"
 #include "variants.h"
 
@@ -348,6 +349,32 @@ int launch_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t
     return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
 }
 
+template <int IN_DT>
+int quantize_t(int mode, QuantArgs &a, hipStream_t stream) {
+    const uint64_t groups = (uint64_t)a.rows * ((a.cols + 3) / 4);
+    if (mode == QGEMM_QUANT_PER_MATRIX) {
+        // two passes: partial maxima (one per workgroup) into the workspace, then scale and cast
+        const uint32_t nblk = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(2048, (groups + 1023) / 1024));
+        void *ws = nullptr;
+        int st = ensure_workspace_locked(nblk * sizeof(float), &ws);
+        if (st != QGEMM_OK) return st;
+        a.partial = (float *)ws;
+        a.npartial = nblk;
+        hipLaunchKernelGGL(quant_amax_kernel<IN_DT>, dim3(nblk), dim3(256), 0, stream, a);
+        const uint32_t nq = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(8192, (groups + 255) / 256));
+        hipLaunchKernelGGL(quant_matrix_kernel<IN_DT>, dim3(nq), dim3(256), 0, stream, a);
+    } else if (mode == QGEMM_QUANT_BLOCK_1x128) {
+        const uint64_t nblocks = (uint64_t)a.rows * ((a.cols + 127) / 128);
+        if ((nblocks + 7) / 8 >= ((uint64_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
+        hipLaunchKernelGGL(quant_row_block_kernel<IN_DT>, dim3((unsigned)((nblocks + 7) / 8)), dim3(256), 0, stream, a);
+    } else {
+        const uint64_t nblocks = (uint64_t)((a.rows + 127) / 128) * ((a.cols + 127) / 128);
+        if (nblocks >= ((uint64_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
+        hipLaunchKernelGGL(quant_square_block_kernel<IN_DT>, dim3((unsigned)nblocks), dim3(256), 0, stream, a);
+    }
+    return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
+}
+
 }  // namespace
 
 // ===========================================================================
@@ -416,6 +443,47 @@ QGEMM_EXPORT int qgemm_last_config(char *buf, size_t buflen) {
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     std::snprintf(buf, buflen, "%s", g_ctx.last_config.c_str());
     return QGEMM_OK;
+}
+
+QGEMM_EXPORT int qgemm_quantize(int in_dtype, int out_dtype, int mode, const void *x, size_t ld, size_t rows, size_t cols,
+                                void *q, size_t ldq, float *scales, size_t scale_rs, size_t scale_cs, void *stream_) {
+    if (in_dtype != QGEMM_DT_F32 && in_dtype != QGEMM_DT_BF16 && in_dtype != QGEMM_DT_F16) return QGEMM_ERR_UNSUPPORTED;
+    if (out_dtype != QGEMM_DT_I8 && out_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
+    if (mode != QGEMM_QUANT_PER_MATRIX && mode != QGEMM_QUANT_BLOCK_1x128 && mode != QGEMM_QUANT_BLOCK_128x128)
+        return QGEMM_ERR_INVALID_ARG;
+    if (mode != QGEMM_QUANT_PER_MATRIX && out_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
+    if (!scales) return QGEMM_ERR_INVALID_ARG;
+    if (rows >= ((size_t)1 << 31) || cols >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    int st = ensure_init_locked();
+    if (st != QGEMM_OK) return st;
+    hipStream_t stream = (hipStream_t)stream_;
+    QuantArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.x = x;
+    a.q = q;
+    a.scales = scales;
+    a.rows = (uint32_t)rows;
+    a.cols = (uint32_t)cols;
+    a.ld = ld;
+    a.ldq = ldq;
+    a.scale_rs = scale_rs;
+    a.scale_cs = scale_cs;
+    a.out_dtype = out_dtype;
+    if (rows == 0 || cols == 0) {
+        if (mode != QGEMM_QUANT_PER_MATRIX) return QGEMM_OK;
+        // the scale of an empty matrix is the scale of a zero matrix: run the passes over nothing
+        a.rows = a.cols = 0;
+    } else if (!x || !q || ld < cols || ldq < cols) {
+        return QGEMM_ERR_INVALID_ARG;
+    }
+    g_ctx.last_config = mode == QGEMM_QUANT_PER_MATRIX ? "quantize_per_matrix"
+                        : (mode == QGEMM_QUANT_BLOCK_1x128 ? "quantize_1x128" : "quantize_128x128");
+    switch (in_dtype) {
+        case QGEMM_DT_F32: return quantize_t<QGEMM_DT_F32>(mode, a, stream);
+        case QGEMM_DT_BF16: return quantize_t<QGEMM_DT_BF16>(mode, a, stream);
+        default: return quantize_t<QGEMM_DT_F16>(mode, a, stream);
+    }
 }
 
 QGEMM_EXPORT int qgemm_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t N, void *stream) {

@@ -38,6 +38,7 @@ SIGNATURES = {
     "qgemm_gemm": (_i, [_i, _i, _i, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp]),
     "qgemm_scaled_gemm": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _i, _vp]),
     "qgemm_transpose": (_i, [_i, _vp, _vp, _sz, _sz, _vp]),
+    "qgemm_quantize": (_i, [_i, _i, _i, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _sz, _sz, _vp]),
     "qgemm_tile_map": (_i, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32),
                             C.POINTER(C.c_uint32)]),
     "qgemm_set_option": (_i, [C.c_char_p, C.c_long]),

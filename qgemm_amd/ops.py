@@ -4,6 +4,7 @@
   int8_mm / bf16_mm            the stubs in src/gemm/sm80_gemm_kernel.cu:4-22
   matrix_transpose(in, out)    src/transpose/transpose.cu:60-74
   gemm(...)                    GEMM_kernel_v*<In, Out> of include/gemm.h:25-66
+  quantize(x, ...)             the Q_A / Q_B of README.md:1 (the reference has no quantiser)
 
 Tensors are torch CUDA(HIP) tensors; only their data pointers and the current
 stream cross the boundary."""
@@ -17,6 +18,7 @@ DT_F32, DT_BF16, DT_F16, DT_I8, DT_F8E4M3, DT_I32 = 0, 1, 2, 3, 4, 5
 B_KN, B_NK = 0, 1
 SCALE_PER_MATRIX, SCALE_BLOCK128 = 1, 2
 LAYOUT_K_CONTIGUOUS, LAYOUT_REFERENCE = 0, 1
+QUANT_PER_MATRIX, QUANT_BLOCK_1x128, QUANT_BLOCK_128x128 = 1, 2, 3
 
 _TORCH_DT = {
     torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16, torch.int8: DT_I8,
@@ -126,3 +128,30 @@ def matrix_transpose(idata, odata, M=None, N=None):
     N = idata.shape[1] if N is None else N
     check(load_library().qgemm_transpose(idata.element_size(), idata.data_ptr(), odata.data_ptr(), M, N, _stream()))
     return odata
+
+
+def quantize(x, out_dtype=torch.float8_e4m3fn, mode=QUANT_PER_MATRIX, rows_contiguous_scales=False):
+    """q, scales = quantise(x): x [rows, cols] fp32 / bf16 / fp16 (row stride free), q [rows, cols] int8 or
+    fp8-e4m3.  scales: [1] for QUANT_PER_MATRIX; [rows, ceil(cols/128)] for QUANT_BLOCK_1x128 (or its
+    transpose, storage [ceil(cols/128), rows], with rows_contiguous_scales: the a_scale arrangement of the
+    reference layout); [ceil(rows/128), ceil(cols/128)] for QUANT_BLOCK_128x128 (transposed likewise)."""
+    _need_gpu(x)
+    assert x.dim() == 2 and x.stride(1) == 1
+    rows, cols = x.shape
+    q = torch.empty((rows, cols), dtype=out_dtype, device=x.device)
+    if mode == QUANT_PER_MATRIX:
+        scales = torch.empty(1, dtype=torch.float32, device=x.device)
+        rs = cs = 0
+    else:
+        nbr = rows if mode == QUANT_BLOCK_1x128 else (rows + 127) // 128
+        nbc = (cols + 127) // 128
+        if rows_contiguous_scales:
+            scales = torch.empty((nbc, nbr), dtype=torch.float32, device=x.device)
+            rs, cs = 1, nbr
+        else:
+            scales = torch.empty((nbr, nbc), dtype=torch.float32, device=x.device)
+            rs, cs = nbc, 1
+    ld = x.stride(0) if rows > 1 else max(cols, 1)          # the stride of a single row is arbitrary
+    check(load_library().qgemm_quantize(_dt(x), _dt(q, True), mode, x.data_ptr(), ld, rows, cols, q.data_ptr(),
+                                        cols, scales.data_ptr(), rs, cs, _stream()))
+    return q, scales
