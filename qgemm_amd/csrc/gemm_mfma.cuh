@@ -329,8 +329,10 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #pragma unroll
             for (int j = 0; j < NLD; ++j)
                 as_raw[j] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (64 * j + kb * p.as_ks) * 4, 0);
+            // (the solo pipeline fetches one step past the end of K: keep that read inside the array)
+            const uint32_t kbc = kb < p.ksteps ? kb : p.ksteps - 1;
 #pragma unroll
-            for (int j = 0; j < NBS; ++j) bs_raw[j] = p.bs[bs_off[j] + kb * p.bs_ks];
+            for (int j = 0; j < NBS; ++j) bs_raw[j] = p.bs[bs_off[j] + kbc * p.bs_ks];
         }
     };
     auto expand_scales = [&]() {               // what fetch_scales brought becomes as_cur / bs_cur
@@ -467,10 +469,13 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 else
                     acc[a][b] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1], acc[a][b]);
             };
-            auto step = [&](int kt, auto guard_tag) {
-                constexpr bool GUARD = decltype(guard_tag)::value;
+            // The last two steps issue their copies (and the last one its scale fetch) past the end of K like
+            // every other step: the buffer range check turns what lies beyond the operand into zeros, the
+            // rest is data nobody reads, and one straight-line loop body serves all steps (a second, guarded
+            // copy of the body cost register spills of its own).
+            auto step = [&](int kt) {
                 const int a_nx = next_buf(a_rd);
-                const bool copies = !GUARD || kt + 2 < nk;
+                constexpr bool copies = true;
                 // block scales of this step (fetched one step ahead) and the fetch for the next one, in front of
                 // this step's copies: by the time they are used nothing older is still in flight
                 // block scales: fetch_scales brings the a_scale rows of step kt+1 (in front of this step's
@@ -479,9 +484,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // MFMA of row a-1, the multiply behind the second MFMA of row a, so two factors are live at a time.
                 constexpr int BEHIND = 2;      // MFMAs between a partial product and its fold
                 v4f part[BEHIND + 1];
-                if constexpr (C::BLOCK_SCALE) {
-                    if (!GUARD || kt + 1 < nk) fetch_scales(kt + 1);
-                }
+                fetch_scales(kt + 1);
                 auto fold = [&](int i) {
                     if constexpr (C::BLOCK_SCALE && !(DBG & 1) && !(DBG & 128)) {
                         const int pa = i / C::TN, pb = i % C::TN;
@@ -494,9 +497,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 for (int a = 0; a < TMs; ++a) {
                     if (a == BR && !(DBG & 64)) {
                         __builtin_amdgcn_sched_barrier(0);
-                        // lgkmcnt(0) and vmcnt(LPT_A) (vmcnt(0) when this step issued no copies)
-                        if (copies) __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A) & 0xF0FF);
-                        else __builtin_amdgcn_s_waitcnt(0x0070);
+                        // lgkmcnt(0) and vmcnt(LPT_A): all but the A copies of this step
+                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A) & 0xF0FF);
                         phase_barrier();
                     }
                     // the side instructions of a row go between its MFMAs, one at a time: a run of them in front
@@ -568,8 +570,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 a_rd = a_nx;
                 a_wr = next_buf(a_wr);
             };
-            typedef std::integral_constant<bool, true> yes_t;
-            typedef std::integral_constant<bool, false> no_t;
             if (nk > 0) {
                 if constexpr (C::BLOCK_SCALE) {
                     fetch_scales(0);
@@ -596,9 +596,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());
                 phase_barrier();
                 int kt = 0;
-                for (; kt + 2 < nk; ++kt) step(kt, no_t{});
-                for (; kt < nk; ++kt) step(kt, yes_t{});
-                __builtin_amdgcn_s_waitcnt(0x0070);      // reads of the last row done before LDS serves the epilogue
+                for (; kt < nk; ++kt) step(kt);
+                __builtin_amdgcn_s_waitcnt(0x0070);      // copies landed, reads done, before LDS serves the epilogue
                 phase_barrier();
                 // the MFMAs above are opaque to the compiler's hazard handling: give the last one its wait states
                 // before the epilogue reads the accumulators
