@@ -45,9 +45,9 @@ static const Variant kTable[] = {
 #if INST_BLOCK   // no block-scaled form of the solo pipeline: the row is an alias, so indices agree across families
     ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, false),
 #else
-    ROWP("256x256_w2x2_solo", 256, 256, 2, 2, LOAD_DMA, PIPE_SOLO, true),
+    ROWP("256x256_w2x2_solo", 256, 256, 2, 2, LOAD_DMA, PIPE_SOLO, false),
 #endif
-    ROWP("256x256_w2x4_solo8", 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, (bool)INST_BLOCK),
+    ROWP("256x256_w2x4_solo8", 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, true),
     // narrow tiles for skinny M: N / 32 workgroups stream disjoint strips of B over the whole of K, so no
     // K split (and no second pass over partial sums) is needed to occupy the CUs
     ROW("128x32_w4x1_dma", 128, 32, 4, 1, LOAD_DMA, true),

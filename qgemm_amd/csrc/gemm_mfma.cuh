@@ -119,7 +119,9 @@ struct GemmCfg {
     // 8).  A workgroup that streams a narrow strip of B (skinny M) otherwise waits one full memory round trip
     // per K step.  The block-scale form keeps two (its scale loads share vmcnt with the copies).
     static constexpr int NSTAGE_FIT = (160 * 1024) / STAGE_BYTES, NSTAGE_CNT = 2 + 63 / LPT;
-    static constexpr int NSTAGE = (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE) ? 2
+    // Only for the small tiles: a 128 x 128 tile with two stages leaves room for two workgroups per CU, which is
+    // worth more to a compute-bound shape than deeper prefetch.
+    static constexpr int NSTAGE = (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE || BM * BN > 64 * 128) ? 2
                                   : (NSTAGE_FIT < NSTAGE_CNT ? (NSTAGE_FIT < 8 ? NSTAGE_FIT : 8)
                                                              : (NSTAGE_CNT < 8 ? NSTAGE_CNT : 8));
     static constexpr int LDS_BYTES = A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES;
