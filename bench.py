@@ -226,6 +226,29 @@ def main():
             gbs = m4 * k4 * (4.0 * passes + 1.0) / ms / 1e6
             extra["quantize_fp8_%s_f32_%dx%d" % (nm, m4, k4)] = {"GBps": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS, "ms": ms}
         del xq
+        # bf16 8192^3 through this library, and the vendor library on the same box in the role cuBLAS plays in
+        # the reference's harness (tests/cuda_benchmark.cpp): torch.matmul (bf16) and torch._scaled_mm (fp8,
+        # the headline operands), both hipBLASLt underneath.  Reported beside, never part of `value`.
+        xb = torch.randn(M, K, device=dev).bfloat16()
+        yb = torch.randn(N, K, device=dev).bfloat16()
+        cb = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        _, ms = _time_launches(lambda: Q.bf16_mm(xb, yb, cb), 20, 3)
+        extra["bf16_%d" % M] = {"tflops": flops / ms / 1e9, "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["bf16"],
+                                "ms": ms, "kernel": Q.last_config()}
+        vendor = {}
+        try:
+            _, ms = _time_launches(lambda: torch.matmul(xb, yb.t(), out=cb), 20, 3)
+            vendor["torch_matmul_bf16_%d" % M] = {"tflops": flops / ms / 1e9, "ms": ms}
+        except Exception as e:                      # a library row that does not run is reported, not hidden
+            vendor["torch_matmul_bf16_%d" % M] = {"error": str(e)[:200]}
+        try:
+            _, ms = _time_launches(lambda: torch._scaled_mm(a_q, b_q.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16),
+                                   20, 3)
+            vendor["torch_scaled_mm_fp8_%d" % M] = {"tflops": flops / ms / 1e9, "ms": ms}
+        except Exception as e:
+            vendor["torch_scaled_mm_fp8_%d" % M] = {"error": str(e)[:200]}
+        extra["vendor_library"] = vendor
+        del xb, yb, cb
         out["extra"] = extra
 
     # ---- CPU baseline beside it (bounded sample), and a parity spot check of the timed kernel against it

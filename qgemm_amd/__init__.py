@@ -4,7 +4,7 @@ The product is the C-ABI library qgemm_amd/libqgemm.so (HIP kernels, declared
 in include/qgemm.h).  This package is the thin Python host side over that ABI:
 torch is used for device memory and streams only.
 """
-from .lib import QgemmError, load_library, library_path  # noqa: F401
+from .lib import QgemmError, load_library, load_torch_extension, library_path  # noqa: F401
 from .ops import (  # noqa: F401
     DT_BF16, DT_F16, DT_F32, DT_F8E4M3, DT_I8, DT_I32,
     LAYOUT_K_CONTIGUOUS, LAYOUT_REFERENCE, QUANT_BLOCK_128x128, QUANT_BLOCK_1x128, QUANT_PER_MATRIX,

@@ -66,6 +66,31 @@ def load_library():
     return lib
 
 
+_torch_ext = None
+
+
+def load_torch_extension():
+    """The module `qgemm_python` (qgemm_amd/qgemm_python*.so, built by csrc/build_torch_ext.py): the
+    torch-facing entry points fp8_mm / int8_mm / bf16_mm the reference's packaging names (setup.py:73).
+    Raises ImportError when it has not been built."""
+    global _torch_ext
+    if _torch_ext is None:
+        import glob
+        import importlib.util
+
+        import torch  # noqa: F401  (its libraries must be loaded first)
+
+        load_library()
+        found = glob.glob(os.path.join(_HERE, "qgemm_python*.so"))
+        if not found:
+            raise ImportError(f"{_HERE}/qgemm_python*.so is missing: run `python qgemm_amd/csrc/build_torch_ext.py` "
+                              "(or __graft_entry__.build())")
+        spec = importlib.util.spec_from_file_location("qgemm_python", found[0])
+        _torch_ext = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(_torch_ext)
+    return _torch_ext
+
+
 def check(status):
     if status != STATUS_OK:
         lib = load_library()

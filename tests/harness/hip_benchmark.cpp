@@ -24,6 +24,7 @@
 #include "gemm.h"
 #include "matrix_transpose.h"
 #include "mix_gemm.h"
+#include "timer.h"
 
 extern "C" {   // CPU oracle, oracle/cpu_ref.c (test infrastructure)
 void ref_fill_pattern(float *out, size_t n, int which);
@@ -227,6 +228,49 @@ static void check_transpose() {
     HIP_OK(hipFree(di)); HIP_OK(hipFree(dout));
 }
 
+// KernelTimer / KernelTimerScoped (include/timer.h) around launches on a stream of their own: the time they
+// publish must agree with a pair of events recorded beside them, the rate must be calc_ops / time, and the
+// completion callback must run exactly once.
+static void check_timers() {
+    const size_t M = 1024, N = 1024, K = 1024;
+    __hip_bfloat16 *dA, *dB;
+    float *dC;
+    HIP_OK(hipMalloc(&dA, M * K * 2)); HIP_OK(hipMalloc(&dB, K * N * 2)); HIP_OK(hipMalloc(&dC, M * N * 4));
+    HIP_OK(hipMemset(dA, 0, M * K * 2)); HIP_OK(hipMemset(dB, 0, K * N * 2));
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1));
+    std::vector<std::shared_ptr<KernelTimer>> timers;
+    float ms = -1.f, gflops = -1.f;
+    int calls = 0;
+    const int reps = 20;
+    Timer wall;
+    {
+        KernelTimerScoped scope(timers, 2 * M * N * K * reps, &ms, &gflops, stream);
+        timers.back()->set_callback([](float, size_t, float *, float *, void *u) { ++*(int *)u; }, &calls);
+        HIP_OK(hipEventRecord(e0, stream));
+        for (int i = 0; i < reps; ++i)
+            qgemm_gemm(QGEMM_DT_BF16, QGEMM_DT_F32, QGEMM_B_KN, dA, K, dB, N, dC, N, M, N, K, stream);
+        HIP_OK(hipEventRecord(e1, stream));
+    }
+    for (auto &t : timers) t->synchronize();
+    timers[0]->synchronize();              // a second wait must not run the callback again
+    const double host_ms = wall.elapsed();
+    float ev_ms = 0.f;
+    HIP_OK(hipEventElapsedTime(&ev_ms, e0, e1));
+    const double want_gflops = 2.0 * M * N * K * reps / (ms * 1e6);
+    const bool ok = timers.size() == 1 && calls == 1 && ms > 0.f && ms >= ev_ms * 0.999f && ms <= ev_ms + 0.5f &&
+                    ms <= host_ms && std::fabs(gflops - want_gflops) <= 1e-3 * want_gflops;
+    std::cout << "KernelTimerScoped: " << std::fixed << std::setprecision(4) << ms << " ms (events " << ev_ms
+              << " ms, host " << host_ms << " ms), " << std::setprecision(1) << gflops << " GFLOP/s, callback x"
+              << calls << ": " << (ok ? "PASS" : "FAIL") << std::endl;
+    if (!ok) ++g_failures;
+    HIP_OK(hipEventDestroy(e0)); HIP_OK(hipEventDestroy(e1));
+    HIP_OK(hipStreamDestroy(stream));
+    HIP_OK(hipFree(dA)); HIP_OK(hipFree(dB)); HIP_OK(hipFree(dC));
+}
+
 int main(int argc, char **argv) {
     const bool quick = argc > 1 && std::string(argv[1]) == "--quick";
     hipDeviceProp_t prop;
@@ -244,6 +288,7 @@ int main(int argc, char **argv) {
     for (const Shape &s : shapes) bench_bf16(s, warmup, runs, 5e-2);
     bench_fp8_block({256, 384, 512}, warmup, runs);
     check_transpose();
+    check_timers();
     blas::blas_destroy();
     std::cout << "\n" << std::string(100, '=') << "\nBenchmark completed! failures=" << g_failures << std::endl;
     return g_failures ? 1 : 0;
