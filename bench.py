@@ -31,11 +31,14 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a plain copy of
 # known size (`--copy-calibration`).  Measured offline (bench.py cannot run under its own
-# profiler); the summary with the commands is profiles/gemm_nt_f8_256x256_solo_8192.md.
-# Keyed by (kernel name, M): None where no counter run exists.
-FETCH_KIB, FETCH_FACTOR = 405700.0, 2.0     # copy of 262144 KiB reads FETCH_SIZE = 131084
-WRITE_KIB, WRITE_FACTOR = 155648.0, 1.0     # copy of 262144 KiB reads WRITE_SIZE = 262144
-MEASURED_TRAFFIC_BYTES = {("256x256_w2x2_solo", 8192): (FETCH_KIB * FETCH_FACTOR + WRITE_KIB * WRITE_FACTOR) * 1024.0}
+# profiler); the summaries with the commands are profiles/gemm_nt_f8_256x256_solo8_8192.md and
+# profiles/gemm_nt_f8_256x256_solo_8192.md.  Keyed by (kernel name, M): None where no counter run exists.
+FETCH_FACTOR = 2.0     # copy of 262144 KiB reads FETCH_SIZE = 131084
+WRITE_FACTOR = 1.0     # copy of 262144 KiB reads WRITE_SIZE = 262144
+MEASURED_TRAFFIC_BYTES = {      # (FETCH_SIZE KiB * factor + WRITE_SIZE KiB * factor) * 1024
+    ("256x256_w2x4_solo8", 8192): (405763.0 * FETCH_FACTOR + 131072.0 * WRITE_FACTOR) * 1024.0,
+    ("256x256_w2x2_solo", 8192): (405700.0 * FETCH_FACTOR + 155648.0 * WRITE_FACTOR) * 1024.0,
+}
 
 
 def _time_launches(fn, steps, warmup):
