@@ -174,6 +174,48 @@ __global__ void __launch_bounds__(256) transpose_bytes_kernel(const uint8_t *__r
 }
 
 // ---------------------------------------------------------------------------
+// 2-byte transpose for shapes with M % 8 == 0, N % 8 == 0 and 16-byte aligned rows (what
+// matrix_transpose<bf16 / fp16> of the reference is called with, src/transpose/transpose.cu:60-74).
+// No LDS: a lane owns an 8 x 8 block.  It loads eight 16-byte row pieces, interleaves the 16-bit halves
+// of vertically adjacent dwords (one v_perm each: 32 per block), and the rest of the transposition is
+// which register goes into which output dword.  Lanes 8g..8g+7 hold eight neighbouring column blocks,
+// so every load instruction reads 128-byte pieces of 8 rows; lanes g, g+8, .. hold neighbouring row
+// blocks, so every store instruction writes 128-byte pieces of 8 output rows.  A wave covers 64 x 64
+// elements, a workgroup of four waves 64 rows x 256 columns.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) transpose_u16_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out,
+                                                            uint32_t M, uint32_t N) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t m = blockIdx.y * 64 + (lane >> 3) * 8;                   // first of this lane's 8 rows
+    const uint32_t n = blockIdx.x * 256 + wave * 64 + (lane & 7) * 8;       // first of its 8 columns
+    if (m >= M || n >= N) return;                                           // blocks are wholly in or out
+    v4i row[8];
+    const uint16_t *src = in + (size_t)m * N + n;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) row[j] = *(const v4i *)(src + (size_t)j * N);
+    // pair[i][k] = columns 2k (low perm) and 2k+1 (high perm) of rows 2i, 2i+1
+    uint32_t lo[4][4], hi[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t a = (uint32_t)row[2 * i][k], b = (uint32_t)row[2 * i + 1][k];
+            lo[i][k] = __builtin_amdgcn_perm(b, a, 0x05040100);     // (a.lo16, b.lo16)
+            hi[i][k] = __builtin_amdgcn_perm(b, a, 0x07060302);     // (a.hi16, b.hi16)
+        }
+    uint16_t *dst = out + (size_t)n * M + m;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const v4i even = {(int)lo[0][k], (int)lo[1][k], (int)lo[2][k], (int)lo[3][k]};
+        const v4i odd = {(int)hi[0][k], (int)hi[1][k], (int)hi[2][k], (int)hi[3][k]};
+        *(v4i *)(dst + (size_t)(2 * k) * M) = even;
+        *(v4i *)(dst + (size_t)(2 * k + 1) * M) = odd;
+    }
+#endif
+}
+
+// ---------------------------------------------------------------------------
 // Split-K second pass: C[m,n] = cast(scale * sum_z part[z][m,n]), z ascending
 // (a fixed order, so results do not depend on scheduling; int32 stays exact).
 // ---------------------------------------------------------------------------

@@ -331,6 +331,12 @@ int launch_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t
                            (uint32_t)M, (uint32_t)N);
         return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
     }
+    if (elem_bytes == 2 && M % 8 == 0 && N % 8 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0) {
+        dim3 g((unsigned)((N + 255) / 256), (unsigned)((M + 63) / 64));
+        hipLaunchKernelGGL(transpose_u16_kernel, g, dim3(256), 0, stream, (const uint16_t *)in, (uint16_t *)out,
+                           (uint32_t)M, (uint32_t)N);
+        return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
+    }
     switch (elem_bytes) {
         case 1:
             hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, dim3(256), 0, stream, (const uint8_t *)in, (uint8_t *)out,

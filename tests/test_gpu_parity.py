@@ -280,11 +280,13 @@ def test_plain_gemm_reference_pattern_inputs():
 
 # ------------------------------------------------------------------ transpose
 @pytest.mark.parametrize("dt", [torch.uint8, torch.int16, torch.float32])
-@pytest.mark.parametrize("shape", [(64, 32), (128, 256), (100, 36), (1, 77), (1024, 1024), (48, 100), (400, 260)])
+@pytest.mark.parametrize("shape", [(64, 32), (128, 256), (100, 36), (1, 77), (1024, 1024), (48, 100), (400, 260),
+                                   (8, 8), (72, 264), (264, 8), (520, 72)])
 def test_transpose(dt, shape):
     M, N = shape
     say("transpose", dt, shape)
-    a = np.random.default_rng(1).integers(0, 256 if dt == torch.uint8 else 30000, size=(M, N))
+    lo, hi = {torch.uint8: (0, 256), torch.int16: (-32768, 32768)}.get(dt, (0, 30000))
+    a = np.random.default_rng(1).integers(lo, hi, size=(M, N))
     x = torch.from_numpy(a).to(dt).cuda()
     y = torch.zeros((N, M), dtype=dt, device="cuda")
     Q.matrix_transpose(x, y)
