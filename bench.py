@@ -204,8 +204,8 @@ def main():
                 "tflops": 2.0 * m5 * n5 * k5 / ms / 1e9, "GBps": nbytes / ms / 1e6,
                 "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS, "ms": ms, "kernel": Q.last_config()}
             del b5s
-        # cfg 4 in the reference's own storage (A is K x M, B is K x N, scales [K/128, M] and [K/128, N/128]):
-        # two byte transposes in front of the same kernel
+        # cfg 4 in the reference's own storage (A is K x M, B is K x N, scales [K/128, M] and [K/128, N/128]): read
+        # as it lies through K-major tiles and transposing LDS reads
         a4r, _ = _quant_fp8(torch.randn(k4, m4, device=dev))
         b4r, _ = _quant_fp8(torch.randn(k4, n4, device=dev))
         as4r = torch.rand(k4 // 128, m4, device=dev) * 1.5 + 0.5
@@ -238,6 +238,12 @@ def main():
         _, ms = _time_launches(lambda: Q.bf16_mm(xb, yb, cb), 20, 3)
         extra["bf16_%d" % M] = {"tflops": flops / ms / 1e9, "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["bf16"],
                                 "ms": ms, "kernel": Q.last_config()}
+        # the same product with B stored K x N (the storage of GEMM_kernel_v1..v5): the kernel reads it as it lies
+        ybt = yb.t().contiguous()
+        _, ms = _time_launches(lambda: Q.gemm(xb, ybt, cb, "kn"), 20, 3)
+        extra["bf16_nn_%d" % M] = {"tflops": flops / ms / 1e9, "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["bf16"],
+                                   "ms": ms, "kernel": Q.last_config()}
+        del ybt
         vendor = {}
         try:
             _, ms = _time_launches(lambda: torch.matmul(xb, yb.t(), out=cb), 20, 3)

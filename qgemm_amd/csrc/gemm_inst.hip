@@ -3,8 +3,13 @@
 // so the families build in parallel.
 #include "variants.h"
 
+#include <type_traits>
+
 #ifndef INST_ARITH
-#error "compile with -DINST_ARITH=... -DINST_BLOCK=... -DINST_FN=..."
+#error "compile with -DINST_ARITH=... -DINST_BLOCK=... -DINST_FN=... [-DINST_KMAJ=1|2|3]"
+#endif
+#ifndef INST_KMAJ
+#define INST_KMAJ 0      // bit 0: A stored K x M, bit 1: B stored K x N (see GemmCfg::KMAJ)
 #endif
 
 namespace qgemm {
@@ -23,10 +28,24 @@ static hipError_t launch_variant(const GemmArgs &a, uint32_t grid, hipStream_t s
     return hipGetLastError();
 }
 
-#define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) != PIPE_SIMPLE>
-#define ROWP(NAME, BM, BN, WM_, WN_, LD, PP, AUTO)                                                    \
-    {NAME, INST_ARITH, (bool)INST_BLOCK, BM, BN, CFG(BM, BN, WM_, WN_, LD, PP)::THREADS,             \
-     CFG(BM, BN, WM_, WN_, LD, PP)::LDS_BYTES, LD, AUTO, &launch_variant<CFG(BM, BN, WM_, WN_, LD, PP)>}
+#define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) != PIPE_SIMPLE, INST_KMAJ>
+
+// A K-major operand needs whole 128-byte panels of its tile side, four waves and the simple pipeline (GemmCfg's
+// static_asserts); rows of the table that cannot have that are aliases of the 128 x 128 row in such a family,
+// so that force_config indices agree across families, and are never picked by the heuristic.
+constexpr int kElemBytes = (INST_ARITH == AR_BF16 || INST_ARITH == AR_F16) ? 2 : 1;
+constexpr bool kmajor_can(int bm, int bn, int nw, int pipe) {
+    return INST_KMAJ == 0 || (pipe == PIPE_SIMPLE && nw % 4 == 0 && (!(INST_KMAJ & 1) || (bm * kElemBytes) % 128 == 0) &&
+                              (!(INST_KMAJ & 2) || (bn * kElemBytes) % 128 == 0));
+}
+template <bool OK, class C, class Fallback>
+static Variant row_of(const char *name, bool auto_ok) {
+    using P = std::conditional_t<OK, C, Fallback>;
+    return Variant{OK ? name : "128x128_w2x2_dma", P::ARITH, P::BLOCK_SCALE, P::BM, P::BN, P::THREADS, P::LDS_BYTES,
+                   P::LOADER, OK && auto_ok, &launch_variant<P>};
+}
+#define ROWP(NAME, BM, BN, WM_, WN_, LD, PP, AUTO) \
+    row_of<kmajor_can(BM, BN, (WM_) * (WN_), PP), CFG(BM, BN, WM_, WN_, LD, PP), CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>(NAME, AUTO)
 #define ROW(NAME, BM, BN, WM_, WN_, LD, AUTO) ROWP(NAME, BM, BN, WM_, WN_, LD, PIPE_SIMPLE, AUTO)
 
 // force_config indexes this table; the heuristic only considers the rows marked auto.

@@ -95,8 +95,15 @@ enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1, PIPE_SOLO = 2 };
 // the A copy of tile k+2 is started two K steps ahead and only the B half of a tile has to
 // land within one step.
 template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int LOADER_ = LOAD_DMA,
-          int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false>
+          int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false, int KMAJ_ = 0>
 struct GemmCfg {
+    // KMAJ: which operands are stored K-major (bit 0: A is K x M with M contiguous, bit 1: B is K x N with N
+    // contiguous) instead of K-contiguous.  A K-major tile keeps its rows of K in LDS and the MFMA fragments
+    // are taken out of it with the transposing LDS reads (ds_read_b64_tr_b8 / _b16).
+    static constexpr int KMAJ = KMAJ_;
+    static constexpr bool KMA = (KMAJ_ & 1) != 0, KMB = (KMAJ_ & 2) != 0;
+    static constexpr int ES = (ARITH_ == AR_BF16 || ARITH_ == AR_F16) ? 2 : 1;   // operand element bytes
+    static constexpr int KE = 128 / ES;                                          // K elements per step
     static constexpr int LOADER = LOADER_;
     static constexpr int PIPE = PIPE_;
     static constexpr int TAIL = TAIL_;
@@ -121,7 +128,7 @@ struct GemmCfg {
     static constexpr int NSTAGE_FIT = (160 * 1024) / STAGE_BYTES, NSTAGE_CNT = 2 + 63 / LPT;
     // Only for the small tiles: a 128 x 128 tile with two stages leaves room for two workgroups per CU, which is
     // worth more to a compute-bound shape than deeper prefetch.
-    static constexpr int NSTAGE = (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE || BM * BN > 64 * 128) ? 2
+    static constexpr int NSTAGE = (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE || BM * BN > 64 * 128 || KMAJ_ != 0) ? 2
                                   : (NSTAGE_FIT < NSTAGE_CNT ? (NSTAGE_FIT < 8 ? NSTAGE_FIT : 8)
                                                              : (NSTAGE_CNT < 8 ? NSTAGE_CNT : 8));
     static constexpr int LDS_BYTES = A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES;
@@ -138,9 +145,19 @@ struct GemmCfg {
     static_assert(PIPE == PIPE_SIMPLE || (RBA * 2) % NW == 0, "A loads must divide evenly over the waves");
     static_assert(PIPE != PIPE_SIMPLE || (TAIL == 0 && !A3), "TAIL and A3 belong to the pipelined variants");
     static_assert(TAIL >= 0 && TAIL < TN, "TAIL counts B-fragment columns");
+    static_assert(KMAJ == 0 || NW % 4 == 0, "K-major tiles: the swizzle of a copy must not depend on the instruction");
+    static_assert((!KMA || (BM * ES) % 128 == 0) && (!KMB || (BN * ES) % 128 == 0),
+                  "K-major tiles are made of whole 128-byte panels");
+    // The compiler makes every transposing LDS read wait for all global->LDS copies in flight (vmcnt(0)): it cannot
+    // tell that they target another buffer.  The simple pipeline issues the next stage's copies behind the reads
+    // of a step, so nothing is in flight there; the pipelined schedules live on copies in flight and would stall.
+    static_assert(KMAJ == 0 || PIPE == PIPE_SIMPLE, "K-major tiles: simple pipeline only");
 };
 
 typedef __attribute__((address_space(3))) void lds_void;
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v2i lds_v2i;
+typedef __attribute__((address_space(3))) v4s lds_v4s;
 
 __device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes) {
     // raw buffer, 32-bit data format word as used for untyped loads on gfx9
@@ -162,6 +179,17 @@ __device__ inline void phase_barrier() {
 
 // 16-byte slot of (row r in 0..15, chunk c in 0..7) inside a 2 KiB row block
 __host__ __device__ inline constexpr int lds_slot(int r, int c) { return 8 * r + ((c + r) & 7); }
+
+// K-major tiles (row = one k, 128 bytes of m or n; panels of KE rows): the 16-byte chunk c of row k sits in
+// slot c ^ kmajor_swz(k).  A transposing read takes, per 16 lanes, 8 rows x 16 bytes (1-byte elements:
+// rows k0 .. k0+7 with k0 a multiple of 8, groups of lanes 16 rows apart) or 4 rows x 32 bytes (2-byte
+// elements: rows k0 .. k0+3, groups 8 rows apart).  Rows two apart share their banks (64 banks x 4 bytes
+// = two 128-byte rows), so the XOR has to separate rows of equal parity inside a group and the two groups
+// of a half wave: bits 1-2 and 4 of k for bytes, bits 1 and 3 for 16-bit elements.
+template <int ES>
+__host__ __device__ inline constexpr int kmajor_swz(int k) {
+    return ES == 1 ? (((k >> 1) & 3) | (((k >> 4) & 1) << 2)) : ((((k >> 1) & 1) << 1) | (((k >> 3) & 1) << 2));
+}
 
 template <int ARITH>
 struct AccT { typedef v4f type; };
@@ -255,10 +283,18 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const uint32_t a_rows = p.M - row0 < (uint32_t)C::BM ? p.M - row0 : C::BM;
     const uint32_t b_rows = p.N - col0 < (uint32_t)C::BN ? p.N - col0 : C::BN;
     const uint32_t kbytes = (uint32_t)nk * C::BKB;
+    // K-major operand: rows are k (stride lda / ldb bytes), the tile starts at column row0 / col0; the range ends
+    // with the last column of the last k row of this K slice.  Columns past M / N inside an earlier row read
+    // the neighbouring row instead (valid memory) and, as above, only feed outputs that are not stored.
+    const uint32_t krows = nk > 0 ? (uint32_t)nk * C::KE : 1;
     const __amdgpu_buffer_rsrc_t ra =
-        make_rsrc(p.A + (size_t)row0 * p.lda + (size_t)kbeg * C::BKB, (a_rows - 1) * p.lda + kbytes);
+        C::KMA ? make_rsrc(p.A + (size_t)kbeg * C::KE * p.lda + (size_t)row0 * C::ES,
+                           (krows - 1) * p.lda + (p.M - row0) * C::ES)
+               : make_rsrc(p.A + (size_t)row0 * p.lda + (size_t)kbeg * C::BKB, (a_rows - 1) * p.lda + kbytes);
     const __amdgpu_buffer_rsrc_t rb =
-        make_rsrc(p.B + (size_t)col0 * p.ldb + (size_t)kbeg * C::BKB, (b_rows - 1) * p.ldb + kbytes);
+        C::KMB ? make_rsrc(p.B + (size_t)kbeg * C::KE * p.ldb + (size_t)col0 * C::ES,
+                           (krows - 1) * p.ldb + (p.N - col0) * C::ES)
+               : make_rsrc(p.B + (size_t)col0 * p.ldb + (size_t)kbeg * C::BKB, (b_rows - 1) * p.ldb + kbytes);
 
     // ---- the LPT load instructions of this wave.  Instruction q = wave + i*NW (0 .. NLOAD-1) covers
     // rows 8*(q & 1) .. +7 of row block q >> 1 and lands at stage + 1024*q.  With NW even, q & 1 =
@@ -269,10 +305,21 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     constexpr int LPT_A0 = C::LPT_A;                                    // loads i < LPT_A0 fetch A, the rest B
     const int ld_r = 8 * (wave & 1) + (lane >> 3);                      // row inside the row block
     const int ld_chunk = ((lane & 7) - ld_r) & 7;                         // rotation: see lds_slot
-    const uint32_t voff_a = ld_r * p.lda + ld_chunk * 16, voff_b = ld_r * p.ldb + ld_chunk * 16;
+    // K-major tile: row block blk holds k rows 16 * (blk % (KE/16)) .. +15 of panel blk / (KE/16) (a panel = 128
+    // bytes of m or n).  Bit 4 of k is bit 0 of blk = bit 1 of the wave number for every instruction of the wave
+    // (NW / 2 and KE / 16 are even), so the swizzled chunk is one VGPR here too.
+    const int ld_chunk_km = (lane & 7) ^ kmajor_swz<C::ES>(ld_r + 16 * ((wave >> 1) & 1));
+    const uint32_t voff_a = ld_r * p.lda + (C::KMA ? ld_chunk_km : ld_chunk) * 16;
+    const uint32_t voff_b = ld_r * p.ldb + (C::KMB ? ld_chunk_km : ld_chunk) * 16;
     auto load_soff = [&](int i, int kt) -> uint32_t {                   // scalar: row block + K step
-        const uint32_t blk = (wave >> 1) + (i < LPT_A0 ? i : i - LPT_A0) * (C::NW / 2);
-        return blk * 16 * (i < LPT_A0 ? p.lda : p.ldb) + (uint32_t)kt * C::BKB;
+        const bool is_a = i < LPT_A0;
+        const uint32_t blk = (wave >> 1) + (is_a ? i : i - LPT_A0) * (C::NW / 2);
+        const uint32_t ld = is_a ? p.lda : p.ldb;
+        if (is_a ? C::KMA : C::KMB) {
+            constexpr uint32_t BPP = C::KE / 16;                        // row blocks per panel
+            return ((uint32_t)kt * C::KE + (blk % BPP) * 16) * ld + (blk / BPP) * 128;
+        }
+        return blk * 16 * ld + (uint32_t)kt * C::BKB;
     };
 
     auto issue_stage = [&](int kt) {       // LOAD_DMA: global -> LDS
@@ -365,11 +412,36 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const int off0 = lds_slot(fr, fg) * 16, off1 = lds_slot(fr, 4 + fg) * 16;
     const int a_blk0 = (wm * C::TM) * 2048;
     const int b_blk0 = (C::RBA + wn * C::TN) * 2048;
+    // K-major tile: the 16 columns of fragment x16 (counted in 16-column units from the tile's first column)
+    // are chunk c of panel pn; the lane's 16 bytes of a half step are k rows 64*half + 16*fg .. +15 (bytes) or
+    // 32*half + 8*fg .. +7 (16-bit), fetched by two transposing reads.  Lane j of a group of 16 supplies the
+    // address of 8 bytes of the group's row j >> 1 (bytes: 2 lanes per 16-byte row piece) or j >> 2 (16-bit: 4
+    // lanes per 32-byte row piece) and receives column j of the block.  Everything lane-dependent is in km_lane;
+    // the chunk of the fragment comes in by XOR (see kmajor_swz), the rest is an immediate offset.
+    const int km_lane = C::ES == 1 ? ((16 * fg + (fr >> 1)) * 128 + 16 * kmajor_swz<1>(16 * fg + (fr >> 1)) + 8 * (fr & 1))
+                                   : ((8 * fg + (fr >> 2)) * 128 +
+                                      16 * (((fr >> 1) & 1) | kmajor_swz<2>(8 * fg + (fr >> 2))) + 8 * (fr & 1));
+    auto frag_km = [&](const char *tile, int x16, int half) {
+        constexpr int PER_PANEL = 8 / C::ES;                            // fragments per 128-byte panel
+        const int pn = x16 / PER_PANEL, c = (x16 % PER_PANEL) * C::ES;
+        const char *q = tile + (pn * C::KE + half * (C::KE / 2)) * 128 + (km_lane ^ (16 * c));
+        if constexpr (C::ES == 1) {
+            const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)q);
+            const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)(q + 8 * 128));
+            return v4i{lo[0], lo[1], hi[0], hi[1]};
+        } else {
+            const v2i lo = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)q));
+            const v2i hi = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)(q + 4 * 128)));
+            return v4i{lo[0], lo[1], hi[0], hi[1]};
+        }
+    };
     auto frag_a = [&](const char *stage, int a, int half) {
-        return *(const v4i *)(stage + a_blk0 + a * 2048 + (half ? off1 : off0));
+        if constexpr (C::KMA) return frag_km(stage, wm * C::TM + a, half);
+        else return *(const v4i *)(stage + a_blk0 + a * 2048 + (half ? off1 : off0));
     };
     auto frag_b = [&](const char *stage, int b, int half) {
-        return *(const v4i *)(stage + b_blk0 + b * 2048 + (half ? off1 : off0));
+        if constexpr (C::KMB) return frag_km(stage + C::RBA * 2048, wn * C::TN + b, half);
+        else return *(const v4i *)(stage + b_blk0 + b * 2048 + (half ? off1 : off0));
     };
 
     // ---- K loop
@@ -817,10 +889,15 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             }
             __syncthreads();                                 // ... and everybody else's; tile kt-1 is fully consumed
             expand_scales();
-            if (kt + NS - 1 < nk) {                          // into the buffer tile kt-1 has just left
-                if constexpr (C::LOADER == LOAD_DMA) issue_stage(kt + NS - 1);
-                else fetch_stage(kt + 1);
-            }
+            auto next_stage = [&]() {                        // into the buffer tile kt-1 has just left
+                if (kt + NS - 1 < nk) {
+                    if constexpr (C::LOADER == LOAD_DMA) issue_stage(kt + NS - 1);
+                    else fetch_stage(kt + 1);
+                }
+            };
+            // K-major tiles: all fragment reads of the step first, the copies behind them (see GemmCfg)
+            constexpr bool READS_FIRST = C::KMAJ != 0 && C::LOADER == LOAD_DMA;
+            if constexpr (!READS_FIRST) next_stage();
             if (kt + 1 < nk) fetch_scales(kt + 1);
             const char *stage = smem + (kt % NS) * C::STAGE_BYTES;
             v4i fa[C::TM][2];
@@ -829,10 +906,25 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 fa[a][0] = frag_a(stage, a, 0);
                 fa[a][1] = frag_a(stage, a, 1);
             }
+            v4i fball[READS_FIRST ? C::TN : 1][2];
+            if constexpr (READS_FIRST) {
+#pragma unroll
+                for (int b = 0; b < C::TN; ++b) {
+                    fball[b][0] = frag_b(stage, b, 0);
+                    fball[b][1] = frag_b(stage, b, 1);
+                }
+                next_stage();
+            }
 #pragma unroll
             for (int b = 0; b < C::TN; ++b) {
-                const v4i fb0 = frag_b(stage, b, 0);
-                const v4i fb1 = frag_b(stage, b, 1);
+                v4i fb0, fb1;
+                if constexpr (READS_FIRST) {
+                    fb0 = fball[b][0];
+                    fb1 = fball[b][1];
+                } else {
+                    fb0 = frag_b(stage, b, 0);
+                    fb1 = frag_b(stage, b, 1);
+                }
 #pragma unroll
                 for (int a = 0; a < C::TM; ++a) {
                     if constexpr (C::BLOCK_SCALE) {

@@ -33,6 +33,7 @@ struct Context {
     long force_split = 0;       // 0 = heuristic
     long force_group_m = 0;     // 0 = default
     long debug_flags = 0;       // GemmArgs::debug
+    long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes
     std::string last_config;
 };
 
@@ -82,7 +83,11 @@ int ensure_workspace_locked(size_t bytes, void **out) {
     return QGEMM_OK;
 }
 
-const Variant *table_for(int arith, bool block, int *count) {
+// kmaj: GemmCfg::KMAJ of the wanted family (0: both operands K-contiguous)
+const Variant *table_for(int arith, bool block, int kmaj, int *count) {
+    if (kmaj == 3) return (block && arith == AR_F8) ? variants_f8_block_tn(count) : nullptr;
+    if (kmaj == 2) return block ? nullptr : (arith == AR_BF16 ? variants_bf16_nn(count) : (arith == AR_F16 ? variants_f16_nn(count) : nullptr));
+    if (kmaj != 0) return nullptr;
     if (block) return arith == AR_F8 ? variants_f8_block(count) : nullptr;
     switch (arith) {
         case AR_I8: return variants_i8(count);
@@ -113,8 +118,10 @@ struct NtProblem {
     bool block;
     const void *A, *B;
     void *C;
-    size_t lda_bytes, ldb_bytes, ldc;   // ldc in elements
+    size_t lda_bytes, ldb_bytes, ldc;   // ldc in elements; lda / ldb: stride between rows of m / n, or, for a
+                                        // K-major operand (kmaj), between rows of k
     size_t M, N, Kbytes;
+    int kmaj;                           // bit 0: A is stored K x M, bit 1: B is stored K x N
     const float *as, *bs;
     uint32_t as_ms, as_ks, bs_ns, bs_ks;
     int out_dtype, per_matrix, split_k;
@@ -125,15 +132,74 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 // Shapes the MFMA kernel takes (pointer alignment is checked separately);
 // everything else goes to the any-shape kernel.
 bool mfma_shape_ok(const NtProblem &q) {
-    return q.Kbytes % 128 == 0 && q.Kbytes > 0 && q.lda_bytes % 16 == 0 && q.ldb_bytes % 16 == 0 &&
-           q.lda_bytes * 256 < ((size_t)1 << 32) && q.ldb_bytes * 256 < ((size_t)1 << 32) &&
+    const size_t es = (q.arith == AR_BF16 || q.arith == AR_F16) ? 2 : 1, krows = q.Kbytes / es;
+    // 32-bit buffer offsets: 256 tile rows of a K-contiguous operand, every k row of a K-major one
+    const bool a_ok = (q.kmaj & 1) ? (krows * q.lda_bytes < ((size_t)1 << 32) && q.lda_bytes >= q.M * es)
+                                   : q.lda_bytes * 256 < ((size_t)1 << 32);
+    const bool b_ok = (q.kmaj & 2) ? (krows * q.ldb_bytes < ((size_t)1 << 32) && q.ldb_bytes >= q.N * es)
+                                   : q.ldb_bytes * 256 < ((size_t)1 << 32);
+    return q.Kbytes % 128 == 0 && q.Kbytes > 0 && q.lda_bytes % 16 == 0 && q.ldb_bytes % 16 == 0 && a_ok && b_ok &&
            q.M < ((size_t)1 << 31) && q.N < ((size_t)1 << 31) && q.ldc < ((size_t)1 << 32);
 }
 
-// Heuristic over the rows marked auto_ok.  Pass 1: the largest tile that still gives
-// every CU a workgroup.  Pass 2 (small problems): the shortest tile that covers
-// min(M, 128) rows, so B is streamed once, and the K split supplies the parallelism.
-int choose_variant(const Variant *tab, int count, size_t M, size_t N, int cus) {
+// Which tile, and how many K slices.
+//
+// M > 128: a cost estimate over the three tiles worth having there (256 x 256 solo, 128 x 128, 64 x 128) and
+// 1 / 2 / 4 / 8 K slices.  Workgroups run in rounds of CUs x (workgroups that fit a CU); a round costs
+// (K steps x time per step + a fixed prologue / epilogue), a last partial round that leaves a 128 x 128
+// workgroup alone on its CU runs its steps faster, and a K split pays a second launch plus the traffic of the
+// partial planes.  The times per 128-byte K step were read off a sweep of every variant over square and oblong
+// shapes from 1024 to 8192 (fp8 and bf16 agree per step; block scales cost about a third more): 1.25 us for the
+// 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.45 us for 64 x 128,
+// 0.36 us for 128 x 32.
+//
+// M <= 128 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
+// workgroup, else the shortest tile that covers the rows; narrow tiles instead of a K split.
+struct TileModel {
+    int bm, bn, per_cu;
+    double step_shared, step_alone, fixed;     // microseconds
+};
+const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0}, {128, 128, 2, 0.85, 0.66, 2.0}, {64, 128, 1, 0.45, 0.45, 1.5},
+                                 {128, 32, 1, 0.36, 0.36, 1.0}};
+
+int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus, bool may_split,
+                   uint32_t *nsplit_out, double *cost_out = nullptr) {
+    int best = -1;
+    double best_t = 0;
+    for (const TileModel &tm : kTileModels) {
+        int vi = -1;
+        for (int i = 0; i < count; ++i)
+            if (tab[i].auto_ok && tab[i].bm == tm.bm && tab[i].bn == tm.bn) vi = i;
+        if (vi < 0) continue;
+        const size_t tiles = ((M + tm.bm - 1) / tm.bm) * ((N + tm.bn - 1) / tm.bn);
+        for (uint32_t ns = 1; ns <= 8; ns *= 2) {
+            if (ns > 1 && (!may_split || ksteps / ns < 4)) break;
+            const size_t wgs = tiles * ns, slots = (size_t)cus * tm.per_cu, steps = (ksteps + ns - 1) / ns;
+            const size_t full = wgs / slots, rem = wgs % slots;
+            const double scale = block ? 1.35 : 1.0;
+            double t = (double)full * (steps * tm.step_shared * scale + tm.fixed);
+            if (rem) t += steps * (rem <= (size_t)cus ? tm.step_alone : tm.step_shared) * scale + tm.fixed;
+            if (ns > 1) t += 4.0 + (double)M * N * 4.0 * (ns + 1) / 3.0e6;
+            if (best < 0 || t < best_t) {
+                best = vi;
+                best_t = t;
+                *nsplit_out = ns;
+            }
+        }
+    }
+    if (cost_out) *cost_out = best_t;
+    return best;
+}
+
+// kmaj: the table is a K-major family, which has no narrow tiles: the estimate then serves every M
+int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
+                   bool may_split, uint32_t *nsplit_out) {
+    *nsplit_out = 0;                                       // 0: no opinion, plan_nt decides
+    if (M > 128 || kmaj) {
+        const int vi = choose_by_cost(tab, count, M, N, ksteps, block, cus, may_split, nsplit_out);
+        if (vi >= 0) return vi;
+        *nsplit_out = 0;
+    }
     const size_t m16 = std::max<size_t>(16, (M + 15) / 16 * 16);
     const size_t target = std::min<size_t>(m16, 128);   // shorter tiles would stream B more than once
     int best = -1;
@@ -155,6 +221,34 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, int cus) {
     return best;
 }
 
+// Should the problem run with these operands read K-major, as they are stored (strides between k rows given)?
+// Yes when the shape fits and the estimate for the K-major family (simple pipeline, two stages, transposing reads:
+// a fifth slower per step) beats the K-contiguous kernel plus the transposes in front of it (a launch of about
+// 5 us and the matrix read and written at about 5 TB/s each).  Large shapes keep the transposes and the
+// pipelined 256 x 256 tile; small and mid-size ones save the launches.
+bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes) {
+    if (!g_ctx.kmajor) return false;
+    q.kmaj = kmaj;
+    q.lda_bytes = lda_bytes;
+    q.ldb_bytes = ldb_bytes;
+    if (!mfma_shape_ok(q)) return false;
+    int count = 0, count_km = 0;
+    const Variant *tab = table_for(q.arith, q.block, 0, &count), *tab_km = table_for(q.arith, q.block, kmaj, &count_km);
+    if (!tab || !tab_km || count != count_km) return false;
+    if (g_ctx.force_config >= 0 && g_ctx.force_config < count) return true;    // forced rows exist in every family
+    const size_t ksteps = q.Kbytes / 128;
+    const bool may_split = q.split_k == 0;
+    uint32_t ns = 0;
+    double t_km = 0, t_nt = 8.0;                    // a skinny K-contiguous launch: about 8 us
+    if (choose_by_cost(tab_km, count_km, q.M, q.N, ksteps, q.block, g_ctx.num_cus, may_split, &ns, &t_km) < 0) return false;
+    if (q.M > 128 && choose_by_cost(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, may_split, &ns, &t_nt) < 0)
+        return false;
+    const double kbytes = (double)q.Kbytes;         // K * element size
+    if (kmaj & 1) t_nt += 5.0 + 2.0 * (double)q.M * kbytes / 5.0e6;
+    if (kmaj & 2) t_nt += 5.0 + 2.0 * (double)q.N * kbytes / 5.0e6;
+    return 1.2 * t_km <= t_nt;
+}
+
 struct Plan {
     const Variant *v = nullptr;
     GemmArgs a;
@@ -164,10 +258,14 @@ struct Plan {
 
 int plan_nt(const NtProblem &q, Plan &pl) {
     int count = 0;
-    const Variant *tab = table_for(q.arith, q.block, &count);
+    const Variant *tab = table_for(q.arith, q.block, q.kmaj, &count);
     if (!tab) return QGEMM_ERR_UNSUPPORTED;
-    int vi = g_ctx.force_config >= 0 && g_ctx.force_config < count ? (int)g_ctx.force_config
-                                                                    : choose_variant(tab, count, q.M, q.N, g_ctx.num_cus);
+    uint32_t model_split = 0;
+    int vi = choose_variant(tab, count, q.M, q.N, q.Kbytes / 128, q.block, q.kmaj, g_ctx.num_cus, q.split_k == 0, &model_split);
+    if (g_ctx.force_config >= 0 && g_ctx.force_config < count) {
+        vi = (int)g_ctx.force_config;
+        model_split = 0;
+    }
     if (vi < 0) return QGEMM_ERR_UNSUPPORTED;
     const Variant &v = tab[vi];
     pl.v = &v;
@@ -195,6 +293,7 @@ int plan_nt(const NtProblem &q, Plan &pl) {
     if (q.split_k > 1) nsplit = (uint32_t)q.split_k;
     else if (q.split_k == 0) {
         if (g_ctx.force_split > 0) nsplit = (uint32_t)g_ctx.force_split;
+        else if (model_split > 0) nsplit = model_split;
         else if (pl.tiles * 2 <= (size_t)g_ctx.num_cus && a.ksteps >= 8) {
             // enough slices to cover the CUs about twice, at least 4 K steps each
             uint32_t want = (uint32_t)((2 * (size_t)g_ctx.num_cus + pl.tiles - 1) / pl.tiles);
@@ -208,6 +307,8 @@ int plan_nt(const NtProblem &q, Plan &pl) {
     pl.split_bytes = nsplit > 1 ? q.M * q.N * 4 * (size_t)nsplit : 0;
     return QGEMM_OK;
 }
+
+const char *kmaj_suffix(int kmaj) { return kmaj == 3 ? "_tn" : (kmaj == 2 ? "_nn" : ""); }
 
 // split_ws: workspace of pl.split_bytes (ignored when the plan does not split)
 int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
@@ -226,7 +327,7 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
         a.vec_store = ((uintptr_t)q.C % vec == 0) && ((q.ldc * ob) % vec == 0);
         if (a.vec_store && (uintptr_t)q.C % 16 == 0 && (q.ldc * ob) % 16 == 0) a.vec_store = 2;
         hipError_t e = v.launch(a, (uint32_t)pl.tiles, stream);
-        g_ctx.last_config = v.name;
+        g_ctx.last_config = std::string(v.name) + kmaj_suffix(q.kmaj);
         return e == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
     }
 
@@ -256,7 +357,7 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
     r.out_dtype = q.out_dtype;
     r.per_matrix_scale = q.per_matrix;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((plane + 255) / 256)), dim3(256), 0, stream, r);
-    g_ctx.last_config = std::string(v.name) + "_splitk" + std::to_string(a.nsplit);
+    g_ctx.last_config = std::string(v.name) + kmaj_suffix(q.kmaj) + "_splitk" + std::to_string(a.nsplit);
     return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
 }
 
@@ -440,6 +541,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "force_split")) g_ctx.force_split = value;
     else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
     else if (!std::strcmp(key, "debug_flags")) g_ctx.debug_flags = value;
+    else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
     else return QGEMM_ERR_INVALID_ARG;
     return QGEMM_OK;
 }
@@ -535,8 +637,14 @@ QGEMM_EXPORT int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const voi
         q.B = B;
         q.ldb_bytes = ldB * eb;
         if (mfma_shape_ok(q) && aligned16(A) && aligned16(B)) return launch_nt(q, stream);
+    } else if (eb == 2 && aligned16(A) && aligned16(B) && kmajor_problem_ok(q, 2, q.lda_bytes, ldB * eb)) {
+        // "NN", 16-bit operands: the kernel takes B as it is stored (K x N), see GemmCfg::KMAJ
+        q.kmaj = 2;
+        q.B = B;
+        q.ldb_bytes = ldB * eb;
+        return launch_nt(q, stream);
     } else if (ldB == N) {
-        // "NN": bring B to N x K through the transpose utility (the route the reference's
+        // "NN" otherwise: bring B to N x K through the transpose utility (the route the reference's
         // v3.1 launcher sketches, sm80_gemm_kernel_v3.1.cu:277-279), then run the NT kernel.
         q.ldb_bytes = K * eb;
         if (mfma_shape_ok(q) && aligned16(A)) {
@@ -632,9 +740,17 @@ QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, 
         q.A = A;
         q.B = B;
         if (mfma_shape_ok(q) && aligned16(A) && aligned16(B)) return launch_nt(q, stream);
+    } else if (block && aligned16(A) && aligned16(B) && kmajor_problem_ok(q, 3, M, N)) {
+        // reference layout, block scales: A is K x M (M contiguous), B is K x N; the kernel reads both as stored
+        q.kmaj = 3;
+        q.A = A;
+        q.B = B;
+        q.lda_bytes = M;
+        q.ldb_bytes = N;
+        return launch_nt(q, stream);
     } else if (mfma_shape_ok(q)) {
-        // reference layout: A is K x M (M contiguous), B is K x N.  Bring both to K-contiguous
-        // through the transpose utility, then run the NT kernel.
+        // reference layout otherwise: bring both to K-contiguous through the transpose utility, then run
+        // the NT kernel.
         Plan pl;
         st = plan_nt(q, pl);
         if (st != QGEMM_OK) return st;

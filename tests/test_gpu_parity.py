@@ -23,6 +23,7 @@ def _reset_options():
     Q.set_option("force_config", -1)
     Q.set_option("force_split", 0)
     Q.set_option("group_m", 0)
+    Q.set_option("kmajor", 1)
 
 
 def test_selftest_layouts():
@@ -187,6 +188,56 @@ def test_fp8_mm_reference_layout():
     assert np.array_equal(tn, ref)
 
 
+@pytest.mark.parametrize("variant", range(N_VARIANTS))
+@pytest.mark.parametrize("shape", [(160, 224, 512), (288, 544, 384)])
+def test_fp8_mm_reference_layout_native_every_variant(variant, shape):
+    """The reference storage (A is K x M, B is K x N, hip_mix_gemm_kernel.cpp:96,111) read as it lies, through
+    the K-major tiles and the transposing LDS reads, for every tile variant; against the oracle, and against
+    the route through the transpose utility (same kernel arithmetic, other summation order inside an MFMA)."""
+    M, N, K = shape
+    say("fp8_mm reference layout, native", shape, "variant", variant)
+    qa, _, qb, _ = fp8_inputs(M, N, K, seed=500 + variant)
+    as_ = R.fill_uniform((M, K // 128), 501, 0.5, 2.0) / np.float32(448)
+    bs = R.fill_uniform(((N + 127) // 128, K // 128), 502, 0.5, 2.0) / np.float32(448)
+    ref = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)
+    a_t = fp8_tensor(np.ascontiguousarray(qa.T)).t()
+    b_t = fp8_tensor(np.ascontiguousarray(qb.T)).t()
+    as_t = dev(np.ascontiguousarray(as_.T)).t()
+    bs_t = dev(np.ascontiguousarray(bs.T)).t()
+    Q.set_option("force_config", variant)
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.fp8_mm(a_t, b_t, as_t, bs_t, c)
+    assert Q.last_config().endswith("_tn"), Q.last_config()
+    assert_close(host(c), ref, what=Q.last_config())
+    Q.set_option("kmajor", 0)
+    c2 = torch.zeros_like(c)
+    Q.fp8_mm(a_t, b_t, as_t, bs_t, c2)
+    assert not Q.last_config().endswith("_tn")
+    assert_close(host(c), host(c2), rtol=1e-4, atol=1e-4, what="native against transposed")
+
+
+def test_fp8_mm_reference_layout_native_exact_and_split():
+    """Small-integer operands and power-of-two scales: every product and sum is exact, so the K-major path has
+    to give the oracle's bits whatever the order inside an MFMA; also with K split over workgroups."""
+    M, N, K = 96, 160, 1024
+    say("fp8_mm reference layout, native, exact")
+    rng = np.random.default_rng(9)
+    a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+    as_ = (2.0 ** rng.integers(-3, 4, size=(M, K // 128))).astype(np.float32)
+    bs = (2.0 ** rng.integers(-3, 4, size=((N + 127) // 128, K // 128))).astype(np.float32)
+    ref = R.gemm_fp8_block(a, b, as_, bs)
+    a_t = fp8_tensor(np.ascontiguousarray(R.encode_fp8(a).T)).t()
+    b_t = fp8_tensor(np.ascontiguousarray(R.encode_fp8(b).T)).t()
+    as_t, bs_t = dev(np.ascontiguousarray(as_.T)).t(), dev(np.ascontiguousarray(bs.T)).t()
+    for split in (0, 2, 4):
+        Q.set_option("force_split", split)
+        c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        Q.fp8_mm(a_t, b_t, as_t, bs_t, c)
+        assert "_tn" in Q.last_config(), Q.last_config()
+        assert np.array_equal(host(c), ref), Q.last_config()
+
+
 def test_fp8_mm_dispatch_errors_like_the_reference():
     """hip_mix_gemm_kernel.cpp:460,485,503: dimensions not divisible by 32 throw."""
     say("fp8_mm errors")
@@ -263,6 +314,49 @@ def test_plain_gemm_16bit(dtype, layout_b, shape):
         # 16-bit output: half an ulp of the output type on top of the accumulation-order slack
         rtol = 2.0 ** -8 if out_dt == torch.bfloat16 else (2.0 ** -10 if out_dt == torch.float16 else 1e-5)
         assert_close(got, ref, rtol=rtol, atol=1e-3, what=f"{Q.last_config()} {out_dt}")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("variant", range(N_VARIANTS))
+def test_plain_gemm_nn_native_every_variant(dtype, variant):
+    """GEMM_kernel_v1..v5 storage (B is K x N, include/gemm.h:25-66) read as it lies through the K-major B tile,
+    every tile variant, ragged M and N, a padded leading dimension of B, against the oracle."""
+    M, N, K, ldB = 200, 264, 320, 272
+    say("plain NN native", dtype, "variant", variant)
+    enc, dec, tdt = ((R.encode_f16, R.decode_f16, torch.float16) if dtype == "f16"
+                     else (R.encode_bf16, R.decode_bf16, torch.bfloat16))
+    ha, hb = enc(R.fill_uniform((M, K), 71 + variant)), enc(R.fill_uniform((K, N), 72))
+    ref = R.gemm_f32acc(dec(ha), dec(hb), "nn")
+    a = dev(ha.view(np.int16)).view(tdt)
+    b_pad = torch.full((K, ldB), 7.0, dtype=tdt, device="cuda")          # columns N .. ldB-1 must never matter
+    b_pad[:, :N] = dev(hb.view(np.int16)).view(tdt)
+    Q.set_option("force_config", variant)
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.gemm(a, b_pad[:, :N], c, "kn")
+    assert Q.last_config().endswith("_nn"), Q.last_config()
+    assert_close(host(c), ref, rtol=1e-5, atol=1e-3, what=Q.last_config())
+    # the route through the transpose utility needs ldB == N
+    Q.set_option("kmajor", 0)
+    c2 = torch.zeros_like(c)
+    Q.gemm(a, b_pad[:, :N].contiguous(), c2, "kn")
+    assert not Q.last_config().endswith("_nn")
+    assert_close(host(c), host(c2), rtol=1e-5, atol=1e-4, what="native against transposed")
+
+
+def test_plain_gemm_nn_native_exact_integers():
+    """Small integers: exact in bf16 and in the fp32 sums, so the bits must match numpy's integer product."""
+    M, N, K = 256, 384, 512
+    say("plain NN native, exact")
+    rng = np.random.default_rng(12)
+    a = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    b = rng.integers(-4, 5, size=(K, N)).astype(np.float32)
+    ref = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    for split in (0, 3):
+        Q.set_option("force_split", split)
+        c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        Q.gemm(torch.from_numpy(a).cuda().bfloat16(), torch.from_numpy(b).cuda().bfloat16(), c, "kn")
+        assert "_nn" in Q.last_config(), Q.last_config()
+        assert np.array_equal(host(c), ref), Q.last_config()
 
 
 def test_plain_gemm_reference_pattern_inputs():
