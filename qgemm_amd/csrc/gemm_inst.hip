@@ -61,12 +61,15 @@ static const Variant kTable[] = {
     ROW("32x128_w1x4_vgpr", 32, 128, 1, 4, LOAD_VGPR, false),
     ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, false),
     ROWP("256x256_w2x4_pingpong", 256, 256, 2, 4, LOAD_DMA, PIPE_PINGPONG, false),
-#if INST_BLOCK   // no block-scaled form of the solo pipeline: the row is an alias, so indices agree across families
+    // The 256 x 256 tile the heuristic uses: fp8 per-matrix runs fastest on the 4-wave solo schedule (a third
+    // fewer LDS reads: 3 % in interleaved runs); int8 and the 16-bit types on the 8-wave one (their 4-wave form
+    // issues half MFMAs a row apart and measures 2 % slower); block scales need the 8-wave form.
+#if INST_BLOCK   // no block-scaled form of the 4-wave solo pipeline: the row is an alias, so indices agree across families
     ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, false),
 #else
-    ROWP("256x256_w2x2_solo", 256, 256, 2, 2, LOAD_DMA, PIPE_SOLO, false),
+    ROWP("256x256_w2x2_solo", 256, 256, 2, 2, LOAD_DMA, PIPE_SOLO, INST_ARITH == AR_F8 && INST_KMAJ == 0),
 #endif
-    ROWP("256x256_w2x4_solo8", 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, true),
+    ROWP("256x256_w2x4_solo8", 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, INST_BLOCK || INST_ARITH != AR_F8),
     // narrow tiles for skinny M: N / 32 workgroups stream disjoint strips of B over the whole of K, so no
     // K split (and no second pass over partial sums) is needed to occupy the CUs
     ROW("128x32_w4x1_dma", 128, 32, 4, 1, LOAD_DMA, true),

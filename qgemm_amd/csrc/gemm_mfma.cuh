@@ -963,61 +963,110 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     constexpr bool EPI_FITS = C::NW * 2 * EPI_BYTES <= C::LDS_BYTES && C::WN >= 32 && 64 % (C::WN * 2 / 16) == 0 && C::WN <= 256;
     if constexpr (C::PIPE == PIPE_SIMPLE && EPI_FITS) __syncthreads();
     const bool wave_tile_full = row0 + wm * C::WM + C::WM <= p.M && col0 + wn * C::WN + C::WN <= p.N;
-    if constexpr (EPI_FITS) if (p.vec_store == 2 && wave_tile_full) {
-        auto run = [&](auto dt_tag) {
-            constexpr int DT = decltype(dt_tag)::value;
-            constexpr int ES = (DT == QGEMM_DT_BF16 || DT == QGEMM_DT_F16) ? 2 : 4;
-            // row pitch: 32 bytes (2-byte outputs, 8-byte writes) or 64 bytes (4-byte outputs, 16-byte
-            // writes) past a multiple of 256, so the 16 rows a write instruction touches spread over all banks
-            constexpr int PITCH = C::WN * ES + (ES == 2 ? 32 : 64);
-            constexpr int LPR = C::WN * ES / 16;          // lanes per row when reading back
-            constexpr int RPP = 64 / LPR;                 // rows per read instruction
-            constexpr int PASSES = 16 / RPP;
-            static_assert(16 * PITCH <= EPI_BYTES && PASSES >= 1, "scratch slab");
-            char *scratch = smem + wave * (2 * EPI_BYTES);
-            const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
-            const int wr_off = (lane & 15) * PITCH + (lane >> 4) * 4 * ES;
-            const size_t c_row_bytes = (size_t)p.ldc * ES;
-            char *cbase = Cz + ((size_t)(row0 + wm * C::WM) * p.ldc + col0 + wn * C::WN) * ES + rd_col;
-            auto write_slab = [&](int a) {
-                char *wr = scratch + (a & 1) * EPI_BYTES + wr_off;
+    // Every accumulator is read in exactly one place (write_slab): the output type is a uniform branch around
+    // the conversion of a slab, and wave tiles that stick out of C or meet unaligned rows take the same way
+    // through the scratch and differ only in how a slab leaves it (element by element, bounds checked).
+    // With the accumulators of a 128 x 128 wave tile pinned in the 256 accumulation registers, several code
+    // paths that each name all of them made the register allocator spill two dozen of them to memory here.
+    if constexpr (EPI_FITS) {
+      const int DT = p.out_dtype;
+      const bool fast = p.vec_store == 2 && wave_tile_full;
+      // the element size of the output is a compile-time constant of the slab code (two copies of it: the
+      // addressing of the scratch depends on it); the type of that size is a uniform branch inside
+      auto run = [&](auto es_tag) {
+        constexpr int ES = decltype(es_tag)::value;
+        // row pitch: 32 bytes (2-byte outputs, 8-byte writes) or 64 bytes (4-byte outputs, 16-byte
+        // writes) past a multiple of 256, so the 16 rows a write instruction touches spread over all banks
+        constexpr int PITCH = C::WN * ES + (ES == 2 ? 32 : 64);
+        constexpr int LPR = C::WN * ES / 16;          // lanes per row when reading back
+        constexpr int RPP = 64 / LPR;                 // rows per read instruction
+        constexpr int PASSES = 16 / RPP;
+        static_assert(16 * PITCH <= EPI_BYTES && PASSES >= 1, "scratch slab");
+        char *scratch = smem + wave * (2 * EPI_BYTES);
+        const int rd_row = lane / LPR, rd_col = (lane % LPR) * 16;
+        const int wr_off = (lane & 15) * PITCH + (lane >> 4) * 4 * ES;
+        const size_t c_row_bytes = (size_t)p.ldc * ES;
+        const uint32_t wrow0 = row0 + wm * C::WM, wcol0 = col0 + wn * C::WN;
+        char *cwave = Cz + ((size_t)wrow0 * p.ldc + wcol0) * ES;
+        // Accumulators pinned in the accumulation registers (4-wave solo pipeline) are fetched from there one
+        // slab at a time; left to itself the compiler moves all 256 of them into vector registers first.
+        constexpr bool ACC_PINNED = C::PIPE == PIPE_SOLO && C::NW == 4;
+        auto acc_tile = [&](int a, int b) {
+            if constexpr (ACC_PINNED) {
+                acc_t t;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    typename std::remove_reference<decltype(t[0])>::type x;
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[a][b][r]));
+                    t[r] = x;
+                }
+                return t;
+            } else {
+                return acc[a][b];
+            }
+        };
+        auto write_slab = [&](int a) {
+            char *wr = scratch + (a & 1) * EPI_BYTES + wr_off;
+            if (ES == 4 && DT == QGEMM_DT_I32) {
+#pragma unroll
+                for (int b = 0; b < C::TN; ++b) *(acc_t *)(wr + b * 16 * 4) = acc_tile(a, b);
+            } else {
+                v4f v[C::TN];
 #pragma unroll
                 for (int b = 0; b < C::TN; ++b) {
-                    if constexpr (DT == QGEMM_DT_I32) {
-                        *(acc_t *)(wr + b * 16 * 4) = acc[a][b];
-                    } else if constexpr (DT == QGEMM_DT_F32) {
-                        v4f v;
+                    const acc_t t = acc_tile(a, b);
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) v[r] = (float)acc[a][b][r] * scale;
-                        *(v4f *)(wr + b * 16 * 4) = v;
-                    } else {
-                        us4 h;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            const float v = (float)acc[a][b][r] * scale;
-                            h[r] = DT == QGEMM_DT_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
-                        }
-                        *(us4 *)(wr + b * 16 * 2) = h;
-                    }
+                    for (int r = 0; r < 4; ++r) v[b][r] = (float)t[r] * scale;
                 }
-            };
-            write_slab(0);
+                if constexpr (ES == 4) {
 #pragma unroll
-            for (int a = 0; a < C::TM; ++a) {
-                if (a + 1 < C::TM) write_slab(a + 1);
-                const char *rd = scratch + (a & 1) * EPI_BYTES + rd_row * PITCH + rd_col;
+                    for (int b = 0; b < C::TN; ++b) *(v4f *)(wr + b * 16 * 4) = v[b];
+                } else if (DT == QGEMM_DT_BF16) {
+#pragma unroll
+                    for (int b = 0; b < C::TN; ++b)
+                        *(us4 *)(wr + b * 16 * 2) = us4{f32_to_bf16_bits(v[b][0]), f32_to_bf16_bits(v[b][1]),
+                                                        f32_to_bf16_bits(v[b][2]), f32_to_bf16_bits(v[b][3])};
+                } else {
+#pragma unroll
+                    for (int b = 0; b < C::TN; ++b)
+                        *(us4 *)(wr + b * 16 * 2) = us4{f32_to_f16_bits(v[b][0]), f32_to_f16_bits(v[b][1]),
+                                                        f32_to_f16_bits(v[b][2]), f32_to_f16_bits(v[b][3])};
+                }
+            }
+        };
+        write_slab(0);
+#pragma unroll
+        for (int a = 0; a < C::TM; ++a) {
+            const char *slab = scratch + (a & 1) * EPI_BYTES;
+            if (fast) {
+                // read slab a back first (its writes were issued a turn ago; the LDS works in order), convert and
+                // write slab a+1 while those reads are in flight, then store
+                const char *rd = slab + rd_row * PITCH + rd_col;
                 v4i v[PASSES];
 #pragma unroll
                 for (int ps = 0; ps < PASSES; ++ps) v[ps] = *(const v4i *)(rd + ps * RPP * PITCH);
+                if (a + 1 < C::TM) write_slab(a + 1);
 #pragma unroll
                 for (int ps = 0; ps < PASSES; ++ps)
-                    *(v4i *)(cbase + (size_t)(a * 16 + rd_row + ps * RPP) * c_row_bytes) = v[ps];
+                    __builtin_nontemporal_store(
+                        v[ps], (v4i *)(cwave + rd_col + (size_t)(a * 16 + rd_row + ps * RPP) * c_row_bytes));
+            } else {
+                if (a + 1 < C::TM) write_slab(a + 1);
+                // any alignment, any overhang: one element per lane and turn
+                for (int e = lane; e < 16 * C::WN; e += 64) {
+                    const int r = e / C::WN, cidx = e % C::WN;
+                    const uint32_t m = wrow0 + a * 16 + r, n = wcol0 + cidx;
+                    if (m >= p.M || n >= p.N) continue;
+                    char *dst = cwave + (size_t)(a * 16 + r) * c_row_bytes + (size_t)cidx * ES;
+                    const char *src = slab + r * PITCH + cidx * ES;
+                    if (ES == 2) *(unsigned short *)dst = *(const unsigned short *)src;
+                    else *(uint32_t *)dst = *(const uint32_t *)src;
+                }
             }
-        };
-        if (p.out_dtype == QGEMM_DT_BF16) run(std::integral_constant<int, QGEMM_DT_BF16>{});
-        else if (p.out_dtype == QGEMM_DT_F16) run(std::integral_constant<int, QGEMM_DT_F16>{});
-        else if (p.out_dtype == QGEMM_DT_F32) run(std::integral_constant<int, QGEMM_DT_F32>{});
-        else run(std::integral_constant<int, QGEMM_DT_I32>{});
+        }
+      };
+      if (DT == QGEMM_DT_BF16 || DT == QGEMM_DT_F16) run(std::integral_constant<int, 2>{});
+      else run(std::integral_constant<int, 4>{});
         if constexpr (DBG & 8) {
             const unsigned long long t3 = dbg_stamp<DBG>();
             if (lane == 0 && !(DBG & 16)) {
