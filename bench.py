@@ -37,7 +37,7 @@ FETCH_FACTOR = 2.0     # copy of 262144 KiB reads FETCH_SIZE = 131084
 WRITE_FACTOR = 1.0     # copy of 262144 KiB reads WRITE_SIZE = 262144
 MEASURED_TRAFFIC_BYTES = {      # (FETCH_SIZE KiB * factor + WRITE_SIZE KiB * factor) * 1024
     ("256x256_w2x4_solo8", 8192): (405763.0 * FETCH_FACTOR + 131072.0 * WRITE_FACTOR) * 1024.0,
-    ("256x256_w2x2_solo", 8192): (405700.0 * FETCH_FACTOR + 155648.0 * WRITE_FACTOR) * 1024.0,
+    ("256x256_w2x2_solo", 8192): (399561.0 * FETCH_FACTOR + 131206.0 * WRITE_FACTOR) * 1024.0,
 }
 
 
