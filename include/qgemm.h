@@ -138,6 +138,15 @@ int qgemm_tile_map(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n, uint32_t gro
 int qgemm_set_option(const char *key, long value);
 int qgemm_last_config(char *buf, size_t buflen);
 
+/* Which kernel configuration the library would run for a problem with dense, 16-byte aligned operands: the name
+ * qgemm_last_config would report after the call ("256x256_w2x2_solo", "128x128_w2x2_dma_tn_splitk2", ...;
+ * "transpose+<name>" when operands stored K-major go through the transpose kernels first).  Nothing is launched
+ * and no device is needed (256 CUs are assumed before qgemm_init).  No reference counterpart: the reference picks
+ * its tile at compile time (src/include/gemm_config.h:30-36).
+ *   scale_mode 0 = plain GEMM (qgemm_gemm), else as for qgemm_scaled_gemm
+ *   k_major    bit 0: A is stored K x M, bit 1: B is stored K x N (2 = QGEMM_B_KN, 3 = QGEMM_LAYOUT_REFERENCE) */
+int qgemm_plan(int in_dtype, int scale_mode, int k_major, size_t M, size_t N, size_t K, char *buf, size_t buflen);
+
 /* Self-check of the MFMA / LDS-DMA lane layouts the kernels assume, run on the
  * current device.  Writes a short report into buf; returns QGEMM_OK when every
  * assumption holds.  (Counterpart of the reference's playground/ layout probes.) */

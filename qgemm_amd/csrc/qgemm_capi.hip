@@ -553,6 +553,51 @@ QGEMM_EXPORT int qgemm_last_config(char *buf, size_t buflen) {
     return QGEMM_OK;
 }
 
+QGEMM_EXPORT int qgemm_plan(int in_dtype, int scale_mode, int k_major, size_t M, size_t N, size_t K, char *buf,
+                            size_t buflen) {
+    if (!buf || buflen == 0 || M == 0 || N == 0 || K == 0 || k_major < 0 || k_major > 3) return QGEMM_ERR_INVALID_ARG;
+    const int arith = arith_of(in_dtype);
+    if (arith < 0) return QGEMM_ERR_UNSUPPORTED;
+    if (scale_mode != 0 && scale_mode != QGEMM_SCALE_PER_MATRIX && scale_mode != QGEMM_SCALE_BLOCK128)
+        return QGEMM_ERR_INVALID_ARG;
+    if (scale_mode == QGEMM_SCALE_BLOCK128 && arith != AR_F8) return QGEMM_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);          // no device call below: 256 CUs are assumed before qgemm_init
+    const size_t eb = (arith == AR_BF16 || arith == AR_F16) ? 2 : 1;
+    NtProblem q;
+    std::memset(&q, 0, sizeof(q));
+    q.arith = arith;
+    q.block = scale_mode == QGEMM_SCALE_BLOCK128;
+    q.M = M;
+    q.N = N;
+    q.Kbytes = K * eb;
+    q.lda_bytes = q.ldb_bytes = K * eb;
+    q.ldc = N;
+    std::string name;
+    if (k_major) {
+        const size_t lda = (k_major & 1) ? M * eb : K * eb, ldb = (k_major & 2) ? N * eb : K * eb;
+        int rows = 0;
+        const bool family = table_for(arith, q.block, k_major, &rows) != nullptr;
+        if (family && kmajor_problem_ok(q, k_major, lda, ldb)) {
+            q.kmaj = k_major;
+            q.lda_bytes = lda;
+            q.ldb_bytes = ldb;
+        } else {
+            name = "transpose+";
+        }
+    }
+    if (!mfma_shape_ok(q)) {
+        std::snprintf(buf, buflen, "strided_any_shape");
+        return QGEMM_OK;
+    }
+    Plan pl;
+    const int st = plan_nt(q, pl);
+    if (st != QGEMM_OK) return st;
+    name += std::string(pl.v->name) + kmaj_suffix(q.kmaj);
+    if (pl.a.nsplit > 1) name += "_splitk" + std::to_string(pl.a.nsplit);
+    std::snprintf(buf, buflen, "%s", name.c_str());
+    return QGEMM_OK;
+}
+
 QGEMM_EXPORT int qgemm_quantize(int in_dtype, int out_dtype, int mode, const void *x, size_t ld, size_t rows, size_t cols,
                                 void *q, size_t ldq, float *scales, size_t scale_rs, size_t scale_cs, void *stream_) {
     if (in_dtype != QGEMM_DT_F32 && in_dtype != QGEMM_DT_BF16 && in_dtype != QGEMM_DT_F16) return QGEMM_ERR_UNSUPPORTED;

@@ -43,6 +43,7 @@ SIGNATURES = {
                             C.POINTER(C.c_uint32)]),
     "qgemm_set_option": (_i, [C.c_char_p, C.c_long]),
     "qgemm_last_config": (_i, [C.c_char_p, _sz]),
+    "qgemm_plan": (_i, [_i, _i, _i, _sz, _sz, _sz, C.c_char_p, _sz]),
     "qgemm_selftest_layouts": (_i, [C.c_char_p, _sz]),
 }
 

@@ -49,6 +49,13 @@ def set_option(key, value):
     check(load_library().qgemm_set_option(key.encode(), int(value)))
 
 
+def plan(in_dtype, scale_mode, k_major, M, N, K):
+    """Name of the kernel configuration the library would choose (no launch, no device needed)."""
+    buf = C.create_string_buffer(128)
+    check(load_library().qgemm_plan(in_dtype, scale_mode, k_major, M, N, K, buf, 128))
+    return buf.value.decode()
+
+
 def last_config():
     buf = C.create_string_buffer(128)
     check(load_library().qgemm_last_config(buf, 128))

@@ -88,3 +88,41 @@ def test_tile_raster_keeps_an_xcd_on_a_compact_cluster():
         rows = {t[0] for t in first}
         cols = {t[1] for t in first}
         assert len(rows) + len(cols) <= 12      # 8 x 4 cluster: 12 panels for 32 tiles
+
+
+def test_plan_names_the_kernel_without_a_device():
+    """qgemm_plan: the tile / pipeline / K-split choice for the five BASELINE configs and for operands stored
+    K-major, from the host (256 CUs assumed).  Pins the heuristic: a change of choice shows up here first."""
+    plan = Q.plan
+    assert plan(Q.DT_F16, 0, 0, 1024, 1024, 1024) == "128x32_w4x1_dma"                       # config 1
+    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4096) == "256x256_w2x4_solo8"    # config 2
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "256x256_w2x2_solo"  # config 3
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8"  # config 4
+    for m, name in ((16, "16x32_w1x2_dma"), (64, "64x32_w4x1_dma"), (128, "128x32_w4x1_dma")):   # config 5
+        assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
+        assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
+    # mid sizes: the cost estimate prefers 128 x 128 tiles while they fit in one round of two per CU
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 1536, 1536, 1536) == "128x128_w2x2_dma"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2560, 2560, 2560) == "128x128_w2x2_dma"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x2_solo"
+    assert plan(Q.DT_BF16, 0, 0, 512, 4096, 4096) == "64x128_w1x4_dma"
+    # operands stored K-major: read as stored where that is cheaper than transposing, else transposed first
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 2048, 2048, 2048) == "128x128_w2x2_dma_tn"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 6144, 4608, 7168) == "transpose+256x256_w2x4_solo8"
+    assert plan(Q.DT_BF16, 0, 2, 1024, 1024, 1024) == "64x128_w1x4_dma_nn"
+    assert plan(Q.DT_BF16, 0, 2, 8192, 8192, 8192) == "transpose+256x256_w2x4_solo8"
+    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 2, 1024, 1024, 1024).startswith("transpose+")   # no K-major int8 family
+    # K not a multiple of 128 bytes: the any-shape kernel
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 100, 100, 100) == "strided_any_shape"
+    # forced rows are honoured, and a forced split shows in the name
+    Q.set_option("force_config", 2)
+    Q.set_option("force_split", 4)
+    try:
+        assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "128x128_w2x2_dma_splitk4"
+    finally:
+        Q.set_option("force_config", -1)
+        Q.set_option("force_split", 0)
+    with pytest.raises(Q.QgemmError):
+        plan(Q.DT_I8, Q.SCALE_BLOCK128, 0, 256, 256, 256)        # block scales are fp8 only
+    with pytest.raises(Q.QgemmError):
+        plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 0, 256, 256)
