@@ -507,18 +507,30 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             v4i fbr[C::TN][2];         // B fragments
             v4i far[RING][2];          // A fragment ring
             int a_rd = 0, a_wr = 2;
-            // block scales of the current step (as_raw / bs_raw hold what fetch_scales brought for the next)
-            int as_rc[NLD], sc_t[2] = {0, 0};
-            float bs_c[NBS], sc[2][NBS];
+            // block scales of the current step (as_raw / bs_raw hold what fetch_scales brought for the next).
+            // as_b[a] = a_scale of row l & 15 of row block a for every lane l: lane l of as_raw[j] holds the scale of
+            // wave-tile row 64 j + l, and each of its four 16-lane rows is spread over the whole wave with three
+            // lane swaps on the vector ALU (v_permlane16_swap: odd rows of one register against even rows of
+            // the other; v_permlane32_swap: upper half against lower half).  The same pick through ds_bpermute
+            // shares the LDS queue, which answers in order, with the fragment reads issued two rows ahead: waiting
+            // for a pick then means waiting for those reads as well (7 % of the K loop on config 4).
+            float as_b[TMs], bs_c[NBS], sc[2][NBS];
             auto rotate_scales = [&]() {
+                if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
-                for (int j = 0; j < NLD; ++j) as_rc[j] = as_raw[j];
+                    for (int j = 0; j < NLD; ++j) {
+                        const unsigned x = (DBG & 256) ? __builtin_bit_cast(unsigned, 1.0f) : (unsigned)as_raw[j];
+                        const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);      // (R0 R0 R2 R2), (R1 R1 R3 R3)
+                        const auto e = __builtin_amdgcn_permlane32_swap(r[0], r[0], false, false);  // all R0, all R2
+                        const auto o = __builtin_amdgcn_permlane32_swap(r[1], r[1], false, false);  // all R1, all R3
+                        const unsigned rows[4] = {e[0], o[0], e[1], o[1]};
 #pragma unroll
-                for (int j = 0; j < NBS; ++j) bs_c[j] = bs_raw[j];
-            };
-            auto pick_scale = [&](const int *raw, int a) {      // a_scale of row l & 15 of row block a
-                if constexpr (DBG & 256) return __builtin_bit_cast(int, 1.0f);
-                else return __builtin_amdgcn_ds_bpermute(bp0 + ((16 * a) & 63) * 4, raw[(16 * a) / 64]);
+                        for (int q = 0; q < 4; ++q)
+                            if (4 * j + q < TMs) as_b[4 * j + q] = __builtin_bit_cast(float, rows[q]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < NBS; ++j) bs_c[j] = bs_raw[j];
+                }
             };
             auto rd_a = [&](int buf, int a, int slot) {
                 if constexpr (DBG & 4) return;
@@ -608,14 +620,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                                 part[i % (BEHIND + 1)] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0],
                                                                far[a % RING][1], v4f{0, 0, 0, 0});
                             side(b);
-                            if (b == 0) {        // cross-lane pick for the next row, a row's worth of MFMAs ahead
-                                if (a + 1 < TMs) sc_t[(a + 1) % 2] = pick_scale(as_rc, a + 1);
-                                else sc_t[0] = pick_scale(as_raw, 0);      // row 0 of the next step
-                            }
                             if (b == 1) {        // factor of this row, first used behind the next MFMA
 #pragma unroll
-                                for (int j = 0; j < NBS; ++j)
-                                    sc[a % 2][j] = __builtin_bit_cast(float, sc_t[a % 2]) * bs_c[j];
+                                for (int j = 0; j < NBS; ++j) sc[a % 2][j] = as_b[a] * bs_c[j];
                             }
                             __builtin_amdgcn_sched_barrier(0);
                             if (i >= BEHIND) fold(i - BEHIND);
@@ -648,7 +655,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 if constexpr (C::BLOCK_SCALE) {
                     fetch_scales(0);
                     rotate_scales();
-                    sc_t[0] = pick_scale(as_rc, 0);
                 }
 #pragma unroll
                 for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
