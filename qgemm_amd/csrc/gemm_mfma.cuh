@@ -875,6 +875,61 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     } else {
         constexpr int NS = C::NSTAGE;
+        // Small tiles with a deep ring (NS >= 4): two K steps per barrier.  A workgroup of these is alone or nearly
+        // alone on its CU and every step is a chain wait -> barrier -> fragment reads -> a handful of MFMAs, about
+        // 0.25 - 0.36 us; taking the steps in pairs pays the barrier and the LDS latency once for two.  Before turn
+        // kt (even) stages 0 .. kt+NS-3 have been issued; stages kt and kt+1 are waited for, everybody leaves the
+        // buffers of kt-2 and kt-1, and stages kt+NS-2 and kt+NS-1 are issued into them.
+        constexpr bool PAIRS = NS >= 4 && C::LOADER == LOAD_DMA && !C::BLOCK_SCALE && C::KMAJ == 0;
+        if constexpr (PAIRS) {
+#pragma unroll
+            for (int j = 0; j < NS - 2; ++j)
+                if (j < nk) issue_stage(j);
+            for (int kt = 0; kt < nk; kt += 2) {
+                if (kt + NS - 2 <= nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 4) * C::LPT));
+                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
+                __syncthreads();
+                if (kt + NS - 2 < nk) issue_stage(kt + NS - 2);
+                if (kt + NS - 1 < nk) issue_stage(kt + NS - 1);
+                const bool two = kt + 1 < nk;
+                const char *st0 = smem + (kt % NS) * C::STAGE_BYTES, *st1 = smem + ((kt + 1) % NS) * C::STAGE_BYTES;
+                v4i fa[2][C::TM][2], fb[2][C::TN][2];
+#pragma unroll
+                for (int a = 0; a < C::TM; ++a) {
+                    fa[0][a][0] = frag_a(st0, a, 0);
+                    fa[0][a][1] = frag_a(st0, a, 1);
+                }
+#pragma unroll
+                for (int b = 0; b < C::TN; ++b) {
+                    fb[0][b][0] = frag_b(st0, b, 0);
+                    fb[0][b][1] = frag_b(st0, b, 1);
+                }
+                if (two) {
+#pragma unroll
+                    for (int a = 0; a < C::TM; ++a) {
+                        fa[1][a][0] = frag_a(st1, a, 0);
+                        fa[1][a][1] = frag_a(st1, a, 1);
+                    }
+#pragma unroll
+                    for (int b = 0; b < C::TN; ++b) {
+                        fb[1][b][0] = frag_b(st1, b, 0);
+                        fb[1][b][1] = frag_b(st1, b, 1);
+                    }
+                }
+#pragma unroll
+                for (int b = 0; b < C::TN; ++b)
+#pragma unroll
+                    for (int a = 0; a < C::TM; ++a)
+                        acc[a][b] = mma128<C::ARITH>(fb[0][b][0], fb[0][b][1], fa[0][a][0], fa[0][a][1], acc[a][b]);
+                if (two) {
+#pragma unroll
+                    for (int b = 0; b < C::TN; ++b)
+#pragma unroll
+                        for (int a = 0; a < C::TM; ++a)
+                            acc[a][b] = mma128<C::ARITH>(fb[1][b][0], fb[1][b][1], fa[1][a][0], fa[1][a][1], acc[a][b]);
+                }
+            }
+        } else {
         if (nk > 0) {
             if constexpr (C::LOADER == LOAD_DMA) {
 #pragma unroll
@@ -948,6 +1003,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // the other stage was last read in iteration kt-1, which every wave left before this one began
                 if (kt + 1 < nk) commit_stage(kt + 1);
             }
+        }
         }
     }
 
