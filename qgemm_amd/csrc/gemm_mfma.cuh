@@ -1,5 +1,6 @@
-// MFMA GEMM kernel for gfx950, "NT" operands: A is M x K, B is N x K, both with
-// K contiguous.  One template covers int8, fp8-e4m3, bf16 and fp16 inputs.
+// MFMA GEMM kernel for gfx950.  Native operands are "NT": A is M x K, B is N x K, both with K
+// contiguous; GemmCfg::KMAJ adds operands stored K x M / K x N (read through the transposing LDS
+// loads).  One template covers int8, fp8-e4m3, bf16 and fp16 inputs.
 //
 // Replaces the device kernels of the reference:
 //   GEMM_kernel_bf16_v1..v5      src/gemm/sm89_gemm_kernel_v{1,2,3,4,5}.cu
@@ -29,7 +30,8 @@
 //     applies on the read side only.)
 //   * Which K bytes a lane group holds does not matter as long as A and B agree:
 //     the contraction index is summed away.
-//   * LDS holds two stages (double buffer).
+//   * LDS holds two stages in the simple pipeline (up to eight for the small tiles), three A and two
+//     B buffers in the pipelined ones.
 //
 // Math
 //   * The B fragment is fed as the first MFMA operand and the A fragment as the
@@ -47,8 +49,8 @@
 namespace qgemm {
 
 struct GemmArgs {
-    const char *A;        // M x K, row stride lda bytes
-    const char *B;        // N x K, row stride ldb bytes
+    const char *A;        // M x K, row stride lda bytes (KMAJ & 1: K x M, stride between k rows)
+    const char *B;        // N x K, row stride ldb bytes (KMAJ & 2: K x N, stride between k rows)
     char *C;              // M x N row-major, ldc elements; split-K: plane z at C + z*split_stride elements
     const float *as;      // per-matrix: 1 float; block: as[m*as_ms + kb*as_ks]
     const float *bs;      // per-matrix: 1 float; block: bs[nb*bs_ns + kb*bs_ks]
@@ -245,7 +247,7 @@ __device__ inline unsigned long long dbg_stamp() {
 // DBG is a measurement aid for kernel bring-up; the library only instantiates DBG = 0.  Bits: 1 skip the
 // MFMAs, 2 skip the global loads, 4 skip the fragment reads, 8 per-workgroup time stamps (32: on the shared
 // 100 MHz clock), 16 per-phase cycle sums (ping-pong), 64 no barrier (solo), 128 no block-scale fold,
-// 256 constant block scales (no fetch, no cross-lane pick).  Results are wrong with any of 1 .. 4, 64 .. 256.
+// 256 constant block scales (no fetch).  Results are wrong with any of 1 .. 4, 64 .. 256.
 template <class C, int DBG = 0>
 __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
@@ -352,9 +354,10 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // lane l fetches the scale of wave-tile row l (and l + 64), one 256-byte request per 64 rows, through a
     // buffer load (rows past M read as 0 or as some other finite scale; they only meet zero operands).  A
     // step later every lane picks the row of each of its A fragments (row l & 15 of row block a) out of
-    // those registers with ds_bpermute.  One load per lane and fragment instead (16 distinct rows per
-    // instruction, every row a request of its own) keeps the texture addresser busy for longer than the
-    // MFMAs of the step take.
+    // those registers: with ds_bpermute in the simple and ping-pong pipelines, with lane swaps on the vector
+    // ALU in the solo pipeline.  One load per lane and fragment instead (16 distinct rows per instruction,
+    // every row a request of its own) keeps the texture addresser busy for longer than the MFMAs of the
+    // step take.
     constexpr int NBS = C::BLOCK_SCALE ? (C::WN + 127) / 128 : 1;
     constexpr int NLD = C::BLOCK_SCALE ? (C::WM + 63) / 64 : 1;
     float as_cur[C::TM], bs_cur[NBS], bs_raw[NBS];
