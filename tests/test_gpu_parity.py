@@ -318,6 +318,34 @@ def test_plain_gemm_16bit(dtype, layout_b, shape):
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("variant", range(N_VARIANTS))
+def test_plain_gemm_16bit_every_variant(dtype, variant):
+    """Every tile variant on 16-bit operands (the big tiles use the 32 x 32 x 16 MFMA and their own fragment and
+    accumulator layouts): small integers, so sums are exact and the bits must equal numpy's integer product,
+    ragged M and N, 16-bit and fp32 outputs."""
+    M, N, K = 300, 328, 384
+    say("plain 16-bit", dtype, "variant", variant)
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    rng = np.random.default_rng(40 + variant)
+    a = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    b = rng.integers(-4, 5, size=(N, K)).astype(np.float32)
+    ref = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)       # |ref| <= 16 * 384: exact in fp32
+    Q.set_option("force_config", variant)
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.gemm(torch.from_numpy(a).cuda().to(tdt), torch.from_numpy(b).cuda().to(tdt), c, "nk")
+    assert np.array_equal(host(c), ref), Q.last_config()
+    # a row-aligned shape takes the vectorised way out; 16-bit output (values up to 2^8 * 24 are exact in neither
+    # type in general: compare against the rounded reference)
+    M2, N2 = 256, 512
+    c2 = torch.zeros((M2, N2), dtype=tdt, device="cuda")
+    a2 = rng.integers(-2, 3, size=(M2, K)).astype(np.float32)
+    b2 = rng.integers(-2, 3, size=(N2, K)).astype(np.float32)
+    Q.gemm(torch.from_numpy(a2).cuda().to(tdt), torch.from_numpy(b2).cuda().to(tdt), c2, "nk")
+    ref2 = torch.from_numpy((a2.astype(np.int64) @ b2.astype(np.int64).T).astype(np.float32)).to(tdt)
+    assert torch.equal(c2.cpu(), ref2), Q.last_config()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("variant", range(N_VARIANTS))
 def test_plain_gemm_nn_native_every_variant(dtype, variant):
     """GEMM_kernel_v1..v5 storage (B is K x N, include/gemm.h:25-66) read as it lies through the K-major B tile,
     every tile variant, ragged M and N, a padded leading dimension of B, against the oracle."""
