@@ -638,7 +638,14 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #pragma unroll
                             for (int b = 0; b < C::TN; ++b) {
                                 mma(a, b, h);
-                                if (h == 0) side(b);
+                                // the side instructions of the row, spread over all its MFMAs (behind every
+                                // second one where a tile takes two: 16-cycle MFMAs leave room for little more
+                                // than one of them with its address arithmetic)
+                                if constexpr (HALVES == 2) {
+                                    if ((h * C::TN + b) % 2 == 0) side((h * C::TN + b) / 2);
+                                } else {
+                                    side(b);
+                                }
                                 // B(kt)[b] is dead: its registers take B(kt+1)[b]
                                 if (a == TMs - 1 && h == HALVES - 1) rd_b(kt + 1, b);
                             }
