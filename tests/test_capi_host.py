@@ -126,3 +126,18 @@ def test_plan_names_the_kernel_without_a_device():
         plan(Q.DT_I8, Q.SCALE_BLOCK128, 0, 256, 256, 256)        # block scales are fp8 only
     with pytest.raises(Q.QgemmError):
         plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 0, 256, 256)
+
+
+def test_c_abi_header_is_plain_c(tmp_path):
+    """include/qgemm.h is the boundary a C, Go (cgo) or Rust (bindgen) caller binds: it has to compile as C99
+    with warnings as errors, without any HIP or C++ header."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use.c"
+    src.write_text('#include "qgemm.h"\nint main(void) { char b[8]; return qgemm_plan(0, 0, 0, 1, 1, 1, b, sizeof b) == 12345; }\n')
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"),
+                    "-c", str(src), "-o", str(tmp_path / "use.o")], check=True)
