@@ -132,12 +132,13 @@ __global__ void __launch_bounds__(256) transpose_kernel(const T *__restrict__ in
 // registers with byte permutes, and writes the four resulting dwords (4 consecutive m of one n)
 // into the LDS tile [n][m]; the tile leaves as 16-byte pieces of output rows, 128 bytes per row.
 // ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(256) transpose_bytes_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
-                                                              uint32_t M, uint32_t N) {
+// One 128 x 128 tile of the byte transpose (tile_m, tile_n in tiles)
+__device__ inline void transpose_bytes_tile(const uint8_t *__restrict__ in, uint8_t *__restrict__ out, uint32_t M,
+                                            uint32_t N, uint32_t tile_m, uint32_t tile_n) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int T = 128, PITCH = T + 16;        // bytes per LDS row
     __shared__ __attribute__((aligned(16))) uint8_t tile[T * PITCH];
-    const uint32_t m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+    const uint32_t m0 = tile_m * T, n0 = tile_n * T;
     const int cg = threadIdx.x & 31, rg = threadIdx.x >> 5;      // 32 column groups of 4 bytes x 8 row groups of 16
     const uint32_t n = n0 + cg * 4;
 #pragma unroll
@@ -171,6 +172,23 @@ __global__ void __launch_bounds__(256) transpose_bytes_kernel(const uint8_t *__r
         if (on < N && om < M) *(v4i *)(out + (size_t)on * M + om) = *(const v4i *)(tile + r * PITCH + piece * 16);
     }
 #endif
+}
+
+__global__ void __launch_bounds__(256) transpose_bytes_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
+                                                              uint32_t M, uint32_t N) {
+    transpose_bytes_tile(in, out, M, N, blockIdx.y, blockIdx.x);
+}
+
+// Two byte transposes in one launch (both operands of the reference fp8 layout: the second launch costs more
+// than either transpose takes on mid-size shapes): workgroups 0 .. tiles0-1 take matrix 0, the rest matrix 1.
+struct Transpose2Args {
+    const uint8_t *in[2];
+    uint8_t *out[2];
+    uint32_t M[2], N[2], tiles_n[2], tiles0;
+};
+__global__ void __launch_bounds__(256) transpose_bytes2_kernel(const Transpose2Args a) {
+    const uint32_t which = blockIdx.x >= a.tiles0 ? 1u : 0u, t = blockIdx.x - (which ? a.tiles0 : 0u);
+    transpose_bytes_tile(a.in[which], a.out[which], a.M[which], a.N[which], t / a.tiles_n[which], t % a.tiles_n[which]);
 }
 
 // ---------------------------------------------------------------------------

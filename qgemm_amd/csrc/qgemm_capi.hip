@@ -223,8 +223,8 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
 
 // Should the problem run with these operands read K-major, as they are stored (strides between k rows given)?
 // Yes when the shape fits and the estimate for the K-major family (simple pipeline, two stages, transposing reads:
-// a fifth slower per step) beats the K-contiguous kernel plus the transposes in front of it (a launch of about
-// 5 us and the matrix read and written at about 5 TB/s each).  Large shapes keep the transposes and the
+// a fifth slower per step) beats the K-contiguous kernel plus the transpose launch in front of it (about 5 us and
+// the matrices read and written at about 5 TB/s).  Large shapes keep the transposes and the
 // pipelined 256 x 256 tile; small and mid-size ones save the launches.
 bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes) {
     if (!g_ctx.kmajor) return false;
@@ -244,8 +244,9 @@ bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes
     if (q.M > 128 && choose_by_cost(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, may_split, &ns, &t_nt) < 0)
         return false;
     const double kbytes = (double)q.Kbytes;         // K * element size
-    if (kmaj & 1) t_nt += 5.0 + 2.0 * (double)q.M * kbytes / 5.0e6;
-    if (kmaj & 2) t_nt += 5.0 + 2.0 * (double)q.N * kbytes / 5.0e6;
+    t_nt += 5.0;                                     // one launch transposes whatever has to be transposed
+    if (kmaj & 1) t_nt += 2.0 * (double)q.M * kbytes / 5.0e6;
+    if (kmaj & 2) t_nt += 2.0 * (double)q.N * kbytes / 5.0e6;
     return 1.2 * t_km <= t_nt;
 }
 
@@ -805,10 +806,25 @@ QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, 
         st = ensure_workspace_locked(split_room + at_bytes + N * K, &ws);
         if (st != QGEMM_OK) return st;
         char *at = (char *)ws + split_room, *bt = at + at_bytes;
-        st = launch_transpose(1, A, at, K, M, stream);
-        if (st != QGEMM_OK) return st;
-        st = launch_transpose(1, B, bt, K, N, stream);
-        if (st != QGEMM_OK) return st;
+        // M, N, K are multiples of 32 here: both matrices qualify for the register-permute byte transpose
+        if (aligned16(A) && aligned16(B) && K < ((size_t)1 << 31)) {
+            Transpose2Args t;
+            t.in[0] = (const uint8_t *)A; t.out[0] = (uint8_t *)at; t.M[0] = (uint32_t)K; t.N[0] = (uint32_t)M;
+            t.in[1] = (const uint8_t *)B; t.out[1] = (uint8_t *)bt; t.M[1] = (uint32_t)K; t.N[1] = (uint32_t)N;
+            const size_t tk = (K + 127) / 128;
+            t.tiles_n[0] = (uint32_t)((M + 127) / 128);
+            t.tiles_n[1] = (uint32_t)((N + 127) / 128);
+            t.tiles0 = (uint32_t)(tk * t.tiles_n[0]);
+            const size_t total = tk * ((size_t)t.tiles_n[0] + t.tiles_n[1]);
+            if (total >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
+            hipLaunchKernelGGL(transpose_bytes2_kernel, dim3((unsigned)total), dim3(256), 0, stream, t);
+            if (hipGetLastError() != hipSuccess) return QGEMM_ERR_LAUNCH;
+        } else {
+            st = launch_transpose(1, A, at, K, M, stream);
+            if (st != QGEMM_OK) return st;
+            st = launch_transpose(1, B, bt, K, N, stream);
+            if (st != QGEMM_OK) return st;
+        }
         q.A = at;
         q.B = bt;
         return run_nt(q, pl, ws, stream);
