@@ -144,7 +144,7 @@ bool mfma_shape_ok(const NtProblem &q) {
 
 // Which tile, and how many K slices.
 //
-// M > 128: a cost estimate over the three tiles worth having there (256 x 256 solo, 128 x 128, 64 x 128) and
+// M > 128: a cost estimate over the four tiles worth having there (256 x 256 solo, 128 x 128, 64 x 128, 128 x 32) and
 // 1 / 2 / 4 / 8 K slices.  Workgroups run in rounds of CUs x (workgroups that fit a CU); a round costs
 // (K steps x time per step + a fixed prologue / epilogue), a last partial round that leaves a 128 x 128
 // workgroup alone on its CU runs its steps faster, and a K split pays a second launch plus the traffic of the
