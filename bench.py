@@ -89,6 +89,55 @@ def cpu_baseline(a_q, b_q, sa, sb, rows):
     }, c
 
 
+# the shapes of the reference's report (TechniqueReport.md:117-121, 151-155) and a few that do not tile evenly
+SWEEP_SHAPES = [(1024, 512, 2048), (2048, 2048, 2048), (4096, 4096, 4096), (8192, 4096, 2048), (8192, 4096, 4096),
+                (8192, 8192, 8192), (6144, 6144, 6144), (6144, 4608, 7168), (4096, 14336, 4096), (4000, 4000, 4096),
+                (512, 4096, 4096), (2048, 2048, 8192)]
+
+
+def vendor_sweep(Q, torch, dev):
+    """Median over eight interleaved blocks of ten launches each, this library and the vendor's in turn (so both see
+    the same clocks), per shape and input type.  Times are microseconds per call as a Python caller sees them on an
+    otherwise idle stream: below about 25 us the vendor figure is torch's dispatch, not its kernel."""
+    def med(fn_a, fn_b, rounds=8, per_block=10):
+        for _ in range(3):
+            fn_a(); fn_b()
+        ta, tb = [], []
+        for _ in range(rounds):
+            ta.append(_time_launches(fn_a, per_block, 0)[1] * 1e3)
+            tb.append(_time_launches(fn_b, per_block, 0)[1] * 1e3)
+        ta.sort(); tb.sort()
+        return ta[rounds // 2], tb[rounds // 2]
+    rows = []
+    for fam in ("fp8", "int8", "bf16"):
+        for (M, N, K) in SWEEP_SHAPES:
+            if fam == "fp8":
+                a, sa = _quant_fp8(torch.randn(M, K, device=dev)); b, sb = _quant_fp8(torch.randn(N, K, device=dev))
+                c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+                ours = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)
+                theirs = lambda: torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+            elif fam == "int8":
+                a, sa = _quant_i8(torch.randn(M, K, device=dev)); b, sb = _quant_i8(torch.randn(N, K, device=dev))
+                c = torch.empty(M, N, dtype=torch.int32, device=dev)
+                ours = lambda: Q.int8_mm(a, b, sa, sb, c)
+                theirs = lambda: torch._int_mm(a, b.t())
+            else:
+                a = torch.randn(M, K, device=dev).bfloat16(); b = torch.randn(N, K, device=dev).bfloat16()
+                c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+                ours = lambda: Q.bf16_mm(a, b, c)
+                theirs = lambda: torch.matmul(a, b.t(), out=c)
+            row = {"type": fam, "M": M, "N": N, "K": K}
+            try:
+                t_ours, t_theirs = med(ours, theirs)
+                row.update({"this_library_us": round(t_ours, 1), "vendor_us": round(t_theirs, 1),
+                            "ratio": round(t_ours / t_theirs, 3), "kernel": Q.last_config()})
+            except Exception as e:                  # a vendor row that does not run is reported, not hidden
+                row["error"] = str(e)[:200]
+            rows.append(row)
+            print("[sweep]", json.dumps(row), file=sys.stderr, flush=True)
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -102,6 +151,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three plain device copies of 256 MiB (the known-size kernel the FETCH_SIZE / "
                          "WRITE_SIZE counters are scaled against) and exit")
+    ap.add_argument("--vendor-sweep", action="store_true",
+                    help="only time this library against the vendor library (torch.matmul, torch._scaled_mm, "
+                         "torch._int_mm) over a list of shapes, interleaved, print one JSON line and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists).", file=sys.stderr)
@@ -123,6 +175,9 @@ def main():
         return 0
     torch.manual_seed(42)                 # seed of the reference harness, tests/includes/test_config.h:64
     dev = "cuda:0"
+    if args.vendor_sweep:
+        print(json.dumps({"vendor_sweep": vendor_sweep(Q, torch, dev)}))
+        return 0
     M = N = K = args.size
 
     # ---- headline: fp8 per-matrix 8192^3 -> bf16

@@ -75,6 +75,14 @@ static const Variant kTable[] = {
     ROW("128x32_w4x1_dma", 128, 32, 4, 1, LOAD_DMA, true),
     ROW("64x32_w4x1_dma", 64, 32, 4, 1, LOAD_DMA, true),
     ROW("16x32_w1x2_dma", 16, 32, 1, 2, LOAD_DMA, true),
+    // 128 x 128 with eight waves in two K groups (GemmCfg::KG) and four stages (128 KiB: one workgroup per CU): for
+    // shapes with no more tiles than CUs, where the two-stage row above would sit alone on its CU
+#if INST_BLOCK || INST_KMAJ      // (no block-scale or K-major form: alias, so indices agree across families)
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+#else
+    row_of<true, GemmCfg<INST_ARITH, false, 128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 4, 2>,
+           CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("128x128_w2x2_k2", true),
+#endif
 };
 
 const Variant *INST_FN(int *count) {

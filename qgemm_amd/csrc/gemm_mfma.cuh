@@ -97,8 +97,15 @@ enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1, PIPE_SOLO = 2 };
 // the A copy of tile k+2 is started two K steps ahead and only the B half of a tile has to
 // land within one step.
 template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int LOADER_ = LOAD_DMA,
-          int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false, int KMAJ_ = 0>
+          int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false, int KMAJ_ = 0, int STAGES_ = 0, int KGROUPS_ = 1>
 struct GemmCfg {
+    // STAGES (simple pipeline, DMA loader): number of LDS stages, 0 = chosen below.
+    // KGROUPS = 2: the workgroup has two sets of WAVES_M x WAVES_N waves; all of them copy, set 0 computes the
+    // even K steps and set 1 the odd ones of the same tile (one barrier per pair of steps), and the two partial
+    // sums meet in LDS before the epilogue.  A tile that is alone on its CU (a shape with no more tiles than CUs)
+    // otherwise reads its fragments and runs its MFMAs in turn, with nothing to overlap either with: two waves
+    // per SIMD working on different K steps do what a second workgroup on the CU would.
+    static constexpr int KG = KGROUPS_;
     // KMAJ: which operands are stored K-major (bit 0: A is K x M with M contiguous, bit 1: B is K x N with N
     // contiguous) instead of K-contiguous.  A K-major tile keeps its rows of K in LDS and the MFMA fragments
     // are taken out of it with the transposing LDS reads (ds_read_b64_tr_b8 / _b16).
@@ -114,7 +121,7 @@ struct GemmCfg {
     static constexpr bool BLOCK_SCALE = BLOCK_SCALE_;
     static constexpr int BM = BM_, BN = BN_, BKB = 128;         // BKB: bytes of K per step
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
-    static constexpr int NW = WAVES_M * WAVES_N;
+    static constexpr int NW = WAVES_M * WAVES_N * KGROUPS_;
     static constexpr int THREADS = NW * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
     static constexpr int TM = WM / 16, TN = WN / 16;            // 16x16 MFMA tiles per wave
@@ -130,10 +137,17 @@ struct GemmCfg {
     static constexpr int NSTAGE_FIT = (160 * 1024) / STAGE_BYTES, NSTAGE_CNT = 2 + 63 / LPT;
     // Only for the small tiles: a 128 x 128 tile with two stages leaves room for two workgroups per CU, which is
     // worth more to a compute-bound shape than deeper prefetch.
-    static constexpr int NSTAGE = (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE || BM * BN > 64 * 128 || KMAJ_ != 0) ? 2
+    static constexpr int NSTAGE = STAGES_ > 0 ? STAGES_
+                                  : (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE || BM * BN > 64 * 128 || KMAJ_ != 0) ? 2
                                   : (NSTAGE_FIT < NSTAGE_CNT ? (NSTAGE_FIT < 8 ? NSTAGE_FIT : 8)
                                                              : (NSTAGE_CNT < 8 ? NSTAGE_CNT : 8));
     static constexpr int LDS_BYTES = A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES;
+    static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && !BLOCK_SCALE && KMAJ_ == 0 && STAGES_ >= 2 &&
+                                   STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
+                  "explicit stage count: simple pipeline, DMA loader, within LDS and the 6-bit counter");
+    static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && !BLOCK_SCALE && KMAJ_ == 0 &&
+                                    NSTAGE >= 4 && NSTAGE % 2 == 0),
+                  "K groups: simple pipeline, DMA loader, an even number (at least four) of stages");
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
     static_assert(NLOAD % NW == 0, "load instructions must divide evenly over the waves");
     static_assert(!BLOCK_SCALE || ARITH == AR_F8, "block scales are defined for fp8 only");
@@ -259,7 +273,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
+    const int kg = wave / (C::WAVES_M * C::WAVES_N);              // K group of this wave (0 unless GemmCfg::KG == 2)
+    const int wave_q = wave % (C::WAVES_M * C::WAVES_N);          // its place in the group
+    const int wm = wave_q / C::WAVES_N, wn = wave_q % C::WAVES_N;
 
     // ---- which tile, which K slice
     uint32_t wg = blockIdx.x, z = 0;
@@ -890,8 +906,44 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         // 0.25 - 0.36 us; taking the steps in pairs pays the barrier and the LDS latency once for two.  Before turn
         // kt (even) stages 0 .. kt+NS-3 have been issued; stages kt and kt+1 are waited for, everybody leaves the
         // buffers of kt-2 and kt-1, and stages kt+NS-2 and kt+NS-1 are issued into them.
-        constexpr bool PAIRS = NS >= 4 && C::LOADER == LOAD_DMA && !C::BLOCK_SCALE && C::KMAJ == 0;
-        if constexpr (PAIRS) {
+        constexpr bool PAIRS = NS >= 4 && C::LOADER == LOAD_DMA && !C::BLOCK_SCALE && C::KMAJ == 0 && C::BM * C::BN <= 64 * 128 &&
+                               C::KG == 1;
+        if constexpr (C::KG == 2) {
+            // The ring as for PAIRS below; of the two stages a turn waits for, this wave's set takes one.  (Two
+            // stages in flight are 64 KiB per CU: at the latency of a copy that misses the L2 that bounds a turn
+            // from below.  Touching the lines of later turns with plain loads, so that the copies would find them
+            // in the L2, was tried and made the loop a quarter slower.)
+#pragma unroll
+            for (int j = 0; j < NS - 2; ++j)
+                if (j < nk) issue_stage(j);
+            for (int kt = 0; kt < nk; kt += 2) {
+                if (kt + NS - 2 <= nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 4) * C::LPT));
+                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                __syncthreads();
+                if (kt + NS - 2 < nk) issue_stage(kt + NS - 2);
+                if (kt + NS - 1 < nk) issue_stage(kt + NS - 1);
+                const int mine = kt + kg;
+                if (mine < nk) {
+                    const char *st = smem + (mine % NS) * C::STAGE_BYTES;
+                    v4i fa[C::TM][2], fb[C::TN][2];
+#pragma unroll
+                    for (int a = 0; a < C::TM; ++a) {
+                        fa[a][0] = frag_a(st, a, 0);
+                        fa[a][1] = frag_a(st, a, 1);
+                    }
+#pragma unroll
+                    for (int b = 0; b < C::TN; ++b) {
+                        fb[b][0] = frag_b(st, b, 0);
+                        fb[b][1] = frag_b(st, b, 1);
+                    }
+#pragma unroll
+                    for (int b = 0; b < C::TN; ++b)
+#pragma unroll
+                        for (int a = 0; a < C::TM; ++a)
+                            acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                }
+            }
+        } else if constexpr (PAIRS) {
 #pragma unroll
             for (int j = 0; j < NS - 2; ++j)
                 if (j < nk) issue_stage(j);
@@ -1033,7 +1085,30 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // simple pipeline needs one more barrier.
     constexpr int EPI_BYTES = 16 * (C::WN * 4 + 64);
     constexpr bool EPI_FITS = C::NW * 2 * EPI_BYTES <= C::LDS_BYTES && C::WN >= 32 && 64 % (C::WN * 2 / 16) == 0 && C::WN <= 256;
-    if constexpr (C::PIPE == PIPE_SIMPLE && EPI_FITS) __syncthreads();
+    if constexpr (C::KG == 2) {
+        // set 1 hands its partial sums to set 0 through LDS (behind the epilogue scratch of set 0) and is done
+        static_assert(EPI_FITS && (C::NW / 2) * 2 * EPI_BYTES + (C::NW / 2) * C::TM * C::TN * 1024 <= C::LDS_BYTES, "partial sums in LDS");
+        char *part = smem + (C::NW / 2) * 2 * EPI_BYTES + wave_q * (C::TM * C::TN * 1024) + lane * 16;
+        __syncthreads();                                   // every fragment read is over
+        if (kg == 1) {
+#pragma unroll
+            for (int a = 0; a < C::TM; ++a)
+#pragma unroll
+                for (int b = 0; b < C::TN; ++b) *(acc_t *)(part + (a * C::TN + b) * 1024) = acc[a][b];
+        }
+        __syncthreads();
+        if (kg == 1) return;
+#pragma unroll
+        for (int a = 0; a < C::TM; ++a)
+#pragma unroll
+            for (int b = 0; b < C::TN; ++b) {
+                const acc_t o = *(const acc_t *)(part + (a * C::TN + b) * 1024);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[a][b][r] += o[r];
+            }
+    } else if constexpr (C::PIPE == PIPE_SIMPLE && EPI_FITS) {
+        __syncthreads();
+    }
     const bool wave_tile_full = row0 + wm * C::WM + C::WM <= p.M && col0 + wn * C::WN + C::WN <= p.N;
     // Every accumulator is read in exactly one place (write_slab): the output type is a uniform branch around
     // the conversion of a slab, and wave tiles that stick out of C or meet unaligned rows take the same way

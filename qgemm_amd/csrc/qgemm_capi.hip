@@ -144,13 +144,14 @@ bool mfma_shape_ok(const NtProblem &q) {
 
 // Which tile, and how many K slices.
 //
-// M > 128: a cost estimate over the four tiles worth having there (256 x 256 solo, 128 x 128, 64 x 128, 128 x 32) and
+// M > 128: a cost estimate over the tiles worth having there (256 x 256 solo, 128 x 128 in two forms, 64 x 128, 128 x 32) and
 // 1 / 2 / 4 / 8 K slices.  Workgroups run in rounds of CUs x (workgroups that fit a CU); a round costs
 // (K steps x time per step + a fixed prologue / epilogue), a last partial round that leaves a 128 x 128
 // workgroup alone on its CU runs its steps faster, and a K split pays a second launch plus the traffic of the
 // partial planes.  The times per 128-byte K step were read off a sweep of every variant over square and oblong
 // shapes from 1024 to 8192 (fp8 and bf16 agree per step; block scales cost about a third more): 1.25 us for the
-// 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.45 us for 64 x 128,
+// 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.52 us for the 128 x 128
+// row with two K groups (one per CU: it only wins where there are no more tiles than CUs), 0.45 us for 64 x 128,
 // 0.36 us for 128 x 32.
 //
 // M <= 128 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
@@ -158,9 +159,13 @@ bool mfma_shape_ok(const NtProblem &q) {
 struct TileModel {
     int bm, bn, per_cu;
     double step_shared, step_alone, fixed;     // microseconds
+    bool deep;                                 // the four-stage row of this tile (one workgroup per CU, K steps in pairs)
 };
-const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0}, {128, 128, 2, 0.85, 0.66, 2.0}, {64, 128, 1, 0.45, 0.45, 1.5},
-                                 {128, 32, 1, 0.36, 0.36, 1.0}};
+const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false}, {128, 128, 2, 0.85, 0.66, 2.0, false},
+                                 {128, 128, 1, 0.52, 0.52, 3.0, true},  {64, 128, 1, 0.45, 0.45, 1.5, false},
+                                 {128, 32, 1, 0.36, 0.36, 1.0, false}};
+// rows of a variant table that own their CU through LDS although the tile is small
+bool is_deep_row(const Variant &v) { return v.bm * v.bn <= 128 * 128 && v.bm == 128 && v.bn == 128 && v.lds_bytes > 64 * 1024; }
 
 int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus, bool may_split,
                    uint32_t *nsplit_out, double *cost_out = nullptr) {
@@ -169,7 +174,7 @@ int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t kst
     for (const TileModel &tm : kTileModels) {
         int vi = -1;
         for (int i = 0; i < count; ++i)
-            if (tab[i].auto_ok && tab[i].bm == tm.bm && tab[i].bn == tm.bn) vi = i;
+            if (tab[i].auto_ok && tab[i].bm == tm.bm && tab[i].bn == tm.bn && is_deep_row(tab[i]) == tm.deep) vi = i;
         if (vi < 0) continue;
         const size_t tiles = ((M + tm.bm - 1) / tm.bm) * ((N + tm.bn - 1) / tm.bn);
         for (uint32_t ns = 1; ns <= 8; ns *= 2) {
@@ -205,7 +210,7 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     int best = -1;
     size_t best_area = 0;
     for (int i = 0; i < count; ++i) {
-        if (!tab[i].auto_ok || (size_t)tab[i].bm > m16 || (size_t)tab[i].bm < target) continue;
+        if (!tab[i].auto_ok || is_deep_row(tab[i]) || (size_t)tab[i].bm > m16 || (size_t)tab[i].bm < target) continue;
         const size_t tiles = ((M + tab[i].bm - 1) / tab[i].bm) * ((N + tab[i].bn - 1) / tab[i].bn);
         const size_t area = (size_t)tab[i].bm * tab[i].bn;
         if (tiles * 4 >= (size_t)cus * 3 && area > best_area) {     // at least three quarters of the CUs get a tile
@@ -215,7 +220,7 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     }
     if (best >= 0) return best;
     for (int i = 0; i < count; ++i) {
-        if (!tab[i].auto_ok || (size_t)tab[i].bm < target) continue;
+        if (!tab[i].auto_ok || is_deep_row(tab[i]) || (size_t)tab[i].bm < target) continue;
         if (best < 0 || tab[i].bm < tab[best].bm) best = i;
     }
     return best;

@@ -101,8 +101,11 @@ def test_plan_names_the_kernel_without_a_device():
     for m, name in ((16, "16x32_w1x2_dma"), (64, "64x32_w4x1_dma"), (128, "128x32_w4x1_dma")):   # config 5
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
         assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
-    # mid sizes: the cost estimate prefers 128 x 128 tiles while they fit in one round of two per CU
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 1536, 1536, 1536) == "128x128_w2x2_dma"
+    # mid sizes: the cost estimate prefers 128 x 128 tiles while they fit in one round of two per CU, and the
+    # form with two K groups per workgroup where there are no more tiles than CUs
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 1536, 1536, 1536) == "128x128_w2x2_k2"
+    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 2048, 2048, 8192) == "128x128_w2x2_k2"
+    assert plan(Q.DT_BF16, 0, 0, 512, 8192, 8192) == "128x128_w2x2_k2"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2560, 2560, 2560) == "128x128_w2x2_dma"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x2_solo"
     assert plan(Q.DT_BF16, 0, 0, 512, 4096, 4096) == "64x128_w1x4_dma"
