@@ -382,7 +382,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const int bp0 = (lane & 15) * 4;
     __amdgpu_buffer_rsrc_t ras = make_rsrc(p.as, 0);
     if constexpr (C::BLOCK_SCALE) {
-        ras = make_rsrc(p.as, p.M * ((p.ksteps * C::BKB + 127) / 128) * 4);
+        // rows contiguous, p.as_ks floats from one K block to the next (p.as_ks > p.M when the rows are part of a
+        // taller matrix)
+        ras = make_rsrc(p.as, ((p.ksteps - 1) * p.as_ks + p.M) * 4);
         as_voff = (row0 + wm * C::WM + lane) * 4;
 #pragma unroll
         for (int j = 0; j < NBS; ++j) {

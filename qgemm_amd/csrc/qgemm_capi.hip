@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <memory>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -33,6 +34,7 @@ struct Context {
     long force_split = 0;       // 0 = heuristic
     long force_group_m = 0;     // 0 = default
     long debug_flags = 0;       // GemmArgs::debug
+    long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes
     std::string last_config;
 };
@@ -260,14 +262,57 @@ struct Plan {
     GemmArgs a;
     size_t tiles = 0;
     size_t split_bytes = 0;   // workspace the K split needs (0 when not split)
+    // Row split: this plan covers rows [0, m_main) of the problem and `rest` the rows below, as a second launch
+    // with a tile of its own (m_main = 0: no split, the plan covers everything).
+    size_t m_main = 0;
+    std::unique_ptr<Plan> rest;
 };
 
-int plan_nt(const NtProblem &q, Plan &pl) {
+// Rows of the problem that the 256 x 256 tile should keep when its tiles do not fill the last round of CUs.
+// 576 tiles on 256 CUs are 2.25 rounds and cost three: the rows of the two full rounds stay, and the rows below
+// go to whatever the estimate likes best for them (smaller tiles, which fill the CUs).  Returns 0 for "do not
+// split": when the estimate of the two launches (plus 6 us for the second) is not at least 3 % below the one.
+size_t rows_for_full_rounds(const Variant *tab, int count, const Variant &v, size_t M, size_t N, size_t ksteps, bool block,
+                            int cus, double t_single) {
+    if (v.bm != 256 || v.bn != 256 || !g_ctx.row_split) return 0;
+    const size_t tn = (N + 255) / 256, tiles = ((M + 255) / 256) * tn, full = tiles / cus;
+    if (full == 0 || tiles % cus == 0) return 0;
+    const size_t m_main = (full * cus / tn) * 256;
+    if (m_main == 0 || m_main + 128 >= M) return 0;          // (the estimate is for more than 128 rows)
+    uint32_t ns = 0;
+    double t_main = 0, t_rest = 0;
+    if (choose_by_cost(tab, count, m_main, N, ksteps, block, cus, false, &ns, &t_main) < 0) return 0;
+    if (choose_by_cost(tab, count, M - m_main, N, ksteps, block, cus, false, &ns, &t_rest) < 0) return 0;
+    return t_main + t_rest + 6.0 < 0.97 * t_single ? m_main : 0;
+}
+
+int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
     int count = 0;
     const Variant *tab = table_for(q.arith, q.block, q.kmaj, &count);
     if (!tab) return QGEMM_ERR_UNSUPPORTED;
     uint32_t model_split = 0;
     int vi = choose_variant(tab, count, q.M, q.N, q.Kbytes / 128, q.block, q.kmaj, g_ctx.num_cus, q.split_k == 0, &model_split);
+    if (may_split_rows && vi >= 0 && g_ctx.force_config < 0 && g_ctx.force_split <= 0 && q.split_k == 0 && model_split <= 1 &&
+        q.M > 128 && q.kmaj == 0) {
+        uint32_t ns = 0;
+        double t_single = 0;
+        if (choose_by_cost(tab, count, q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, false, &ns, &t_single) == vi) {
+            const size_t m_main = rows_for_full_rounds(tab, count, tab[vi], q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, t_single);
+            if (m_main) {
+                NtProblem q_main = q, q_rest = q;
+                q_main.M = m_main;
+                q_rest.M = q.M - m_main;
+                int st = plan_nt(q_main, pl, false);
+                if (st != QGEMM_OK) return st;
+                pl.rest.reset(new Plan());
+                st = plan_nt(q_rest, *pl.rest, false);
+                if (st != QGEMM_OK) return st;
+                pl.m_main = m_main;
+                pl.split_bytes = std::max(pl.split_bytes, pl.rest->split_bytes);     // one after the other on the stream
+                return QGEMM_OK;
+            }
+        }
+    }
     if (g_ctx.force_config >= 0 && g_ctx.force_config < count) {
         vi = (int)g_ctx.force_config;
         model_split = 0;
@@ -318,10 +363,32 @@ const char *kmaj_suffix(int kmaj) { return kmaj == 3 ? "_tn" : (kmaj == 2 ? "_nn
 
 // split_ws: workspace of pl.split_bytes (ignored when the plan does not split)
 int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
+    if (pl.rest) {
+        // rows [0, m_main) with this plan, the rows below with the other: operands, scales and C move down m_main rows
+        NtProblem q_main = q, q_rest = q;
+        q_main.M = pl.m_main;
+        q_rest.M = q.M - pl.m_main;
+        q_rest.A = (const char *)q.A + pl.m_main * q.lda_bytes;            // (K-contiguous operands only: plan_nt)
+        q_rest.C = (char *)q.C + pl.m_main * q.ldc * dtype_bytes(q.out_dtype);
+        if (q.block && q.as) q_rest.as = q.as + pl.m_main * q.as_ms;
+        std::unique_ptr<Plan> rest = std::move(pl.rest);
+        int st = run_nt(q_main, pl, split_ws, stream);
+        const std::string first = g_ctx.last_config;
+        if (st == QGEMM_OK) st = run_nt(q_rest, *rest, split_ws, stream);
+        g_ctx.last_config = first + "+" + g_ctx.last_config;
+        pl.rest = std::move(rest);
+        return st;
+    }
     const Variant &v = *pl.v;
     GemmArgs &a = pl.a;
     a.A = (const char *)q.A;
     a.B = (const char *)q.B;
+    a.as = q.as;
+    a.bs = q.bs;
+    a.as_ms = q.as_ms;
+    a.as_ks = q.as_ks;
+    a.bs_ns = q.bs_ns;
+    a.bs_ks = q.bs_ks;
     const bool i32_acc = q.arith == AR_I8;
     if (a.nsplit == 1) {
         a.C = (char *)q.C;
@@ -400,11 +467,8 @@ int launch_nt(NtProblem q, hipStream_t stream) {
         if (st != QGEMM_OK) return st;
     }
     if (as_room) {
-        st = scales_rows_contiguous(q, (char *)ws + split_room, stream);
+        st = scales_rows_contiguous(q, (char *)ws + split_room, stream);      // (run_nt takes the scales from q)
         if (st != QGEMM_OK) return st;
-        pl.a.as = q.as;
-        pl.a.as_ms = q.as_ms;
-        pl.a.as_ks = q.as_ks;
     }
     return run_nt(q, pl, ws, stream);
 }
@@ -548,6 +612,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
     else if (!std::strcmp(key, "debug_flags")) g_ctx.debug_flags = value;
     else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
+    else if (!std::strcmp(key, "row_split")) g_ctx.row_split = value;
     else return QGEMM_ERR_INVALID_ARG;
     return QGEMM_OK;
 }
@@ -600,6 +665,10 @@ QGEMM_EXPORT int qgemm_plan(int in_dtype, int scale_mode, int k_major, size_t M,
     if (st != QGEMM_OK) return st;
     name += std::string(pl.v->name) + kmaj_suffix(q.kmaj);
     if (pl.a.nsplit > 1) name += "_splitk" + std::to_string(pl.a.nsplit);
+    if (pl.rest) {
+        name += "+" + std::string(pl.rest->v->name);
+        if (pl.rest->a.nsplit > 1) name += "_splitk" + std::to_string(pl.rest->a.nsplit);
+    }
     std::snprintf(buf, buflen, "%s", name.c_str());
     return QGEMM_OK;
 }

@@ -20,6 +20,7 @@ def _reset_options():
     yield
     Q.set_option("force_config", -1)
     Q.set_option("force_split", 0)
+    Q.set_option("row_split", 1)
 
 
 def _sample(n, count, seed):
@@ -152,3 +153,56 @@ def test_cfg5_skinny_split_k(M):
     assert_close(host(cb), fref, what=Q.last_config())
     Q.scaled_gemm(fp8_tensor(fa), fp8_tensor(fb), scalar(ta), scalar(tb), cb, M, N, K, Q.SCALE_PER_MATRIX, split_k=4)
     assert_close(host(cb), fref, what=Q.last_config())
+
+
+def test_row_split_of_a_partly_empty_last_round():
+    """4608 x 7680 are 540 tiles of 256 x 256 on 256 CUs: the rows of the two full rounds (4352) go to the 256 x 256
+    kernel, the 256 rows below to a second launch with smaller tiles.  int8: the same integers as the single
+    launch, everywhere, and the oracle's on sampled rows on both sides of the seam; fp8 block-scaled and bf16:
+    within tolerance of the oracle on rows of both parts, and of the single launch everywhere."""
+    M, N, K = 4608, 7680, 2048
+    M1 = 4352
+    say("row split int8", M, N, K)
+    assert "+" in Q.plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, M, N, K)
+    rng = np.random.default_rng(21)
+    qa = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    qb = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    da, db_ = dev(qa), dev(qb)
+    c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    Q.int8_mm(da, db_, scalar(1.0), scalar(1.0), c)
+    name = Q.last_config()
+    assert "+" in name, name
+    rows = np.concatenate([_sample(M1, 12, 5), M1 + _sample(M - M1, 12, 6), [M1 - 1, M1, M - 1]])
+    assert np.array_equal(host(c)[rows], R.gemm_i8_i32(qa[rows], qb)), name
+    Q.set_option("row_split", 0)
+    c1 = torch.zeros_like(c)
+    Q.int8_mm(da, db_, scalar(1.0), scalar(1.0), c1)
+    assert "+" not in Q.last_config() and torch.equal(c, c1)
+    Q.set_option("row_split", 1)
+
+    say("row split fp8 block-scaled", M, N, K)
+    qa8, _ = R.quantize_fp8(R.fill_normal((M, K), 31))
+    qb8, _ = R.quantize_fp8(R.fill_normal((N, K), 32))
+    as_ = R.fill_uniform((M, K // 128), 33, 0.5, 2.0) / np.float32(448)
+    bs = R.fill_uniform((N // 128, K // 128), 34, 0.5, 2.0) / np.float32(448)
+    cb = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa8), fp8_tensor(qb8), dev(as_), dev(bs), cb, M, N, K, Q.SCALE_BLOCK128)
+    name = Q.last_config()
+    assert "+" in name, name
+    ref = R.gemm_fp8_block(R.decode_fp8(qa8[rows]), R.decode_fp8(qb8), as_[rows], bs)
+    assert_close(host(cb)[rows], ref, what=name)
+    Q.set_option("row_split", 0)
+    cb1 = torch.zeros_like(cb)
+    Q.scaled_gemm(fp8_tensor(qa8), fp8_tensor(qb8), dev(as_), dev(bs), cb1, M, N, K, Q.SCALE_BLOCK128)
+    assert "+" not in Q.last_config()
+    assert torch.all((cb1.float() - cb.float()).abs() <= 2.0 ** -7 * cb.float().abs() + 1e-3)
+    Q.set_option("row_split", 1)
+
+    say("row split bf16", M, N, K)
+    ha, hb = R.encode_bf16(R.fill_uniform((M, K), 41)), R.encode_bf16(R.fill_uniform((N, K), 42))
+    a16, b16 = dev(ha.view(np.int16)).view(torch.bfloat16), dev(hb.view(np.int16)).view(torch.bfloat16)
+    c16 = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.gemm(a16, b16, c16, "nk")
+    name = Q.last_config()
+    assert "+" in name, name
+    assert_close(host(c16)[rows], R.gemm_f32acc(R.decode_bf16(ha[rows]), R.decode_bf16(hb)), rtol=1e-4, atol=1e-3, what=name)
