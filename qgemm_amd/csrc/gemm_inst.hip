@@ -83,6 +83,13 @@ static const Variant kTable[] = {
     row_of<true, GemmCfg<INST_ARITH, false, 128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 4, 2>,
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("128x128_w2x2_k2", true),
 #endif
+    // the same for the 64 x 128 tile, with six stages (two turns of copies in flight)
+#if INST_BLOCK || INST_KMAJ
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+#else
+    row_of<true, GemmCfg<INST_ARITH, false, 64, 128, 1, 4, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 6, 2>,
+           CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("64x128_w1x4_k2", true),
+#endif
 };
 
 const Variant *INST_FN(int *count) {

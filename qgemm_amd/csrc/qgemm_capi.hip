@@ -161,13 +161,13 @@ bool mfma_shape_ok(const NtProblem &q) {
 struct TileModel {
     int bm, bn, per_cu;
     double step_shared, step_alone, fixed;     // microseconds
-    bool deep;                                 // the four-stage row of this tile (one workgroup per CU, K steps in pairs)
+    bool kgroups;                              // the row of this tile with two K groups per workgroup (GemmCfg::KG)
 };
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false}, {128, 128, 2, 0.85, 0.66, 2.0, false},
                                  {128, 128, 1, 0.52, 0.52, 3.0, true},  {64, 128, 1, 0.45, 0.45, 1.5, false},
-                                 {128, 32, 1, 0.36, 0.36, 1.0, false}};
-// rows of a variant table that own their CU through LDS although the tile is small
-bool is_deep_row(const Variant &v) { return v.bm * v.bn <= 128 * 128 && v.bm == 128 && v.bn == 128 && v.lds_bytes > 64 * 1024; }
+                                 {64, 128, 1, 0.42, 0.42, 2.5, true},   {128, 32, 1, 0.36, 0.36, 1.0, false}};
+// rows with two K groups: eight waves on a tile that otherwise has four
+bool is_deep_row(const Variant &v) { return v.bm * v.bn <= 128 * 128 && v.threads == 512 && (v.bn == 128) && (v.bm == 128 || v.bm == 64); }
 
 int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus, bool may_split,
                    uint32_t *nsplit_out, double *cost_out = nullptr) {
@@ -176,7 +176,7 @@ int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t kst
     for (const TileModel &tm : kTileModels) {
         int vi = -1;
         for (int i = 0; i < count; ++i)
-            if (tab[i].auto_ok && tab[i].bm == tm.bm && tab[i].bn == tm.bn && is_deep_row(tab[i]) == tm.deep) vi = i;
+            if (tab[i].auto_ok && tab[i].bm == tm.bm && tab[i].bn == tm.bn && is_deep_row(tab[i]) == tm.kgroups) vi = i;
         if (vi < 0) continue;
         const size_t tiles = ((M + tm.bm - 1) / tm.bm) * ((N + tm.bn - 1) / tm.bn);
         for (uint32_t ns = 1; ns <= 8; ns *= 2) {
