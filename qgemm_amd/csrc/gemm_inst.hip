@@ -62,8 +62,9 @@ static const Variant kTable[] = {
     ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, false),
     ROWP("256x256_w2x4_pingpong", 256, 256, 2, 4, LOAD_DMA, PIPE_PINGPONG, false),
     // The 256 x 256 tile the heuristic uses: fp8 per-matrix runs fastest on the 4-wave solo schedule (a third
-    // fewer LDS reads: 3 % in interleaved runs); int8 and the 16-bit types on the 8-wave one (their 4-wave form
-    // issues half MFMAs a row apart and measures 2 % slower); block scales need the 8-wave form.
+    // fewer LDS reads: 3 % in interleaved runs); for int8 and the 16-bit types the table marks the 8-wave one and
+    // choose_variant swaps in the 4-wave one where the tiles fill whole rounds of CUs (1 % faster there, 1 - 6 %
+    // slower in partly filled rounds); block scales need the 8-wave form.
 #if INST_BLOCK   // no block-scaled form of the 4-wave solo pipeline: the row is an alias, so indices agree across families
     ROWP("256x256_w4x2_pingpong", 256, 256, 4, 2, LOAD_DMA, PIPE_PINGPONG, false),
 #else

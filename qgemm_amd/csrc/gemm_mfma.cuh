@@ -490,17 +490,30 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         constexpr int B_BASE = NA_BUF * C::A_BYTES;
         constexpr int LPT_A = C::LPT_A, LPT_B = C::LPT - C::LPT_A;
         // instruction i < LPT_A of this wave belongs to A, the rest to B (RBA*2 % NW == 0)
+        // 4-wave solo pipeline: the row-block part of a copy's address sits in a vector register per copy (there
+        // are registers to spare) and the scalar offset is the K step alone, one register for all 16 copies of a
+        // step; with one wave per SIMD every scalar add between two MFMAs is issue time the MFMAs do not get.
+        constexpr bool VOFF_PER_COPY = C::PIPE == PIPE_SOLO && C::NW == 4 && C::KMAJ == 0;
+        uint32_t vo_copy[VOFF_PER_COPY ? C::LPT : 1];
+        if constexpr (VOFF_PER_COPY) {
+#pragma unroll
+            for (int i = 0; i < C::LPT; ++i) vo_copy[i] = (i < LPT_A ? voff_a : voff_b) + load_soff(i, 0);
+        }
         auto issue_a1 = [&](int i, int kt, int buf) {
             if constexpr (DBG & 2) return;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                ra, (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024), 16, voff_a,
-                load_soff(i, kt), 0, 0);
+            lds_void *dst = (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024);
+            if constexpr (VOFF_PER_COPY)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, vo_copy[i], (uint32_t)kt * C::BKB, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, load_soff(i, kt), 0, 0);
         };
         auto issue_b1 = [&](int i, int kt) {
             if constexpr (DBG & 2) return;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                rb, (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (wave + i * C::NW) * 1024 - C::A_BYTES), 16,
-                voff_b, load_soff(i, kt), 0, 0);
+            lds_void *dst = (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (wave + i * C::NW) * 1024 - C::A_BYTES);
+            if constexpr (VOFF_PER_COPY)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vo_copy[i], (uint32_t)kt * C::BKB, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, load_soff(i, kt), 0, 0);
         };
         auto next_buf = [&](int bufi) { return bufi + 1 == NA_BUF ? 0 : bufi + 1; };
         if constexpr (C::PIPE == PIPE_SOLO) {

@@ -203,8 +203,21 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
                    bool may_split, uint32_t *nsplit_out) {
     *nsplit_out = 0;                                       // 0: no opinion, plan_nt decides
     if (M > 128 || kmaj) {
-        const int vi = choose_by_cost(tab, count, M, N, ksteps, block, cus, may_split, nsplit_out);
-        if (vi >= 0) return vi;
+        int vi = choose_by_cost(tab, count, M, N, ksteps, block, cus, may_split, nsplit_out);
+        if (vi >= 0) {
+            // 256 x 256, int8 and 16-bit types: the 8-wave form needs fewer cycles per tile, the 4-wave form a third
+            // fewer LDS reads.  When the tiles fill whole rounds of CUs the part runs at its power limit and the
+            // 4-wave form wins by 1 % (higher clock); in a partly filled round the clock is not what limits and the
+            // 8-wave form wins by 1 - 6 %.  (fp8 per-matrix: the 4-wave form either way; block scales: 8 waves.)
+            const Variant &v = tab[vi];
+            const size_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+            if (v.bm == 256 && v.bn == 256 && v.threads == 512 && !block && kmaj == 0 && *nsplit_out <= 1 && tiles % cus == 0)
+                for (int i = 0; i < count; ++i)
+                    if (tab[i].bm == 256 && tab[i].bn == 256 && tab[i].threads == 256 && tab[i].lds_bytes == v.lds_bytes &&
+                        !std::strcmp(tab[i].name, "256x256_w2x2_solo"))
+                        vi = i;
+            return vi;
+        }
         *nsplit_out = 0;
     }
     const size_t m16 = std::max<size_t>(16, (M + 15) / 16 * 16);

@@ -95,7 +95,10 @@ def test_plan_names_the_kernel_without_a_device():
     K-major, from the host (256 CUs assumed).  Pins the heuristic: a change of choice shows up here first."""
     plan = Q.plan
     assert plan(Q.DT_F16, 0, 0, 1024, 1024, 1024) == "128x32_w4x1_dma"                       # config 1
-    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4096) == "256x256_w2x4_solo8"    # config 2
+    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4096) == "256x256_w2x2_solo"     # config 2
+    # int8 and 16-bit types: 4 waves when the tiles fill whole rounds of CUs, 8 waves in a partly filled round
+    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x4_solo8"
+    assert plan(Q.DT_BF16, 0, 0, 8192, 4096, 4096) == "256x256_w2x2_solo"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "256x256_w2x2_solo"  # config 3
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8"  # config 4
     for m, name in ((16, "16x32_w1x2_dma"), (64, "64x32_w4x1_dma"), (128, "128x32_w4x1_dma")):   # config 5
@@ -113,7 +116,7 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 2048, 2048, 2048) == "128x128_w2x2_dma_tn"
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 6144, 4608, 7168) == "transpose+256x256_w2x4_solo8"
     assert plan(Q.DT_BF16, 0, 2, 1024, 1024, 1024) == "64x128_w1x4_dma_nn"
-    assert plan(Q.DT_BF16, 0, 2, 8192, 8192, 8192) == "transpose+256x256_w2x4_solo8"
+    assert plan(Q.DT_BF16, 0, 2, 8192, 8192, 8192) == "transpose+256x256_w2x2_solo"
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 2, 1024, 1024, 1024).startswith("transpose+")   # no K-major int8 family
     # K not a multiple of 128 bytes: the any-shape kernel
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 100, 100, 100) == "strided_any_shape"
