@@ -167,7 +167,7 @@ const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false}, {128, 12
                                  {128, 128, 1, 0.52, 0.52, 3.0, true},  {64, 128, 1, 0.45, 0.45, 1.5, false},
                                  {64, 128, 1, 0.42, 0.42, 2.5, true},   {128, 32, 1, 0.36, 0.36, 1.0, false}};
 // rows with two K groups: eight waves on a tile that otherwise has four
-bool is_deep_row(const Variant &v) { return v.bm * v.bn <= 128 * 128 && v.threads == 512 && (v.bn == 128) && (v.bm == 128 || v.bm == 64); }
+bool is_kgroup_row(const Variant &v) { return v.bm * v.bn <= 128 * 128 && v.threads == 512 && (v.bn == 128) && (v.bm == 128 || v.bm == 64); }
 
 int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus, bool may_split,
                    uint32_t *nsplit_out, double *cost_out = nullptr) {
@@ -176,7 +176,7 @@ int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t kst
     for (const TileModel &tm : kTileModels) {
         int vi = -1;
         for (int i = 0; i < count; ++i)
-            if (tab[i].auto_ok && tab[i].bm == tm.bm && tab[i].bn == tm.bn && is_deep_row(tab[i]) == tm.kgroups) vi = i;
+            if (tab[i].auto_ok && tab[i].bm == tm.bm && tab[i].bn == tm.bn && is_kgroup_row(tab[i]) == tm.kgroups) vi = i;
         if (vi < 0) continue;
         const size_t tiles = ((M + tm.bm - 1) / tm.bm) * ((N + tm.bn - 1) / tm.bn);
         for (uint32_t ns = 1; ns <= 8; ns *= 2) {
@@ -225,7 +225,7 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     int best = -1;
     size_t best_area = 0;
     for (int i = 0; i < count; ++i) {
-        if (!tab[i].auto_ok || is_deep_row(tab[i]) || (size_t)tab[i].bm > m16 || (size_t)tab[i].bm < target) continue;
+        if (!tab[i].auto_ok || is_kgroup_row(tab[i]) || (size_t)tab[i].bm > m16 || (size_t)tab[i].bm < target) continue;
         const size_t tiles = ((M + tab[i].bm - 1) / tab[i].bm) * ((N + tab[i].bn - 1) / tab[i].bn);
         const size_t area = (size_t)tab[i].bm * tab[i].bn;
         if (tiles * 4 >= (size_t)cus * 3 && area > best_area) {     // at least three quarters of the CUs get a tile
@@ -235,7 +235,7 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     }
     if (best >= 0) return best;
     for (int i = 0; i < count; ++i) {
-        if (!tab[i].auto_ok || is_deep_row(tab[i]) || (size_t)tab[i].bm < target) continue;
+        if (!tab[i].auto_ok || is_kgroup_row(tab[i]) || (size_t)tab[i].bm < target) continue;
         if (best < 0 || tab[i].bm < tab[best].bm) best = i;
     }
     return best;
