@@ -42,7 +42,7 @@ template <bool OK, class C, class Fallback>
 static Variant row_of(const char *name, bool auto_ok) {
     using P = std::conditional_t<OK, C, Fallback>;
     return Variant{OK ? name : "128x128_w2x2_dma", P::ARITH, P::BLOCK_SCALE, P::BM, P::BN, P::THREADS, P::LDS_BYTES,
-                   P::LOADER, OK && auto_ok, &launch_variant<P>};
+                   P::LOADER, OK && auto_ok, P::KG, &launch_variant<P>};
 }
 #define ROWP(NAME, BM, BN, WM_, WN_, LD, PP, AUTO) \
     row_of<kmajor_can(BM, BN, (WM_) * (WN_), PP), CFG(BM, BN, WM_, WN_, LD, PP), CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>(NAME, AUTO)

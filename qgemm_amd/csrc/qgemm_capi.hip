@@ -166,8 +166,8 @@ struct TileModel {
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false}, {128, 128, 2, 0.85, 0.66, 2.0, false},
                                  {128, 128, 1, 0.52, 0.52, 3.0, true},  {64, 128, 1, 0.45, 0.45, 1.5, false},
                                  {64, 128, 1, 0.42, 0.42, 2.5, true},   {128, 32, 1, 0.36, 0.36, 1.0, false}};
-// rows with two K groups: eight waves on a tile that otherwise has four
-bool is_kgroup_row(const Variant &v) { return v.bm * v.bn <= 128 * 128 && v.threads == 512 && (v.bn == 128) && (v.bm == 128 || v.bm == 64); }
+// rows with two K groups: eight waves on a tile that otherwise has four (one workgroup per CU)
+bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 
 int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus, bool may_split,
                    uint32_t *nsplit_out, double *cost_out = nullptr) {
