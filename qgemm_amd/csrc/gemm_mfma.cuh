@@ -494,26 +494,59 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         // are registers to spare) and the scalar offset is the K step alone, one register for all 16 copies of a
         // step; with one wave per SIMD every scalar add between two MFMAs is issue time the MFMAs do not get.
         constexpr bool VOFF_PER_COPY = C::PIPE == PIPE_SOLO && C::NW == 4 && C::KMAJ == 0;
+        // ... and a wave's copies are neighbours in LDS (instruction q = wave * LPT_A + i of the A list, likewise
+        // for B; elsewhere q = wave + i * NW), so that four of them share one LDS base in M0 and differ in the
+        // instruction's immediate offset (0 .. 3072).  The hardware adds that immediate to the global address as
+        // well: the descriptors of these kernels start GROUP_SPAN bytes below the tile and every vector offset
+        // carries GROUP_SPAN minus its immediate, so no offset is negative and the range check sees the same sums.
+        constexpr int GROUP_SPAN = 3072;
+        static_assert(!VOFF_PER_COPY || (LPT_A % 4 == 0 && LPT_B % 4 == 0), "copies go in groups of four");
         uint32_t vo_copy[VOFF_PER_COPY ? C::LPT : 1];
+        __amdgpu_buffer_rsrc_t ra_g = ra, rb_g = rb;
         if constexpr (VOFF_PER_COPY) {
+            const uint32_t a_rows_ = p.M - row0 < (uint32_t)C::BM ? p.M - row0 : C::BM;
+            const uint32_t b_rows_ = p.N - col0 < (uint32_t)C::BN ? p.N - col0 : C::BN;
+            ra_g = make_rsrc(p.A + (size_t)row0 * p.lda + (size_t)kbeg * C::BKB - GROUP_SPAN, (a_rows_ - 1) * p.lda + kbytes + GROUP_SPAN);
+            rb_g = make_rsrc(p.B + (size_t)col0 * p.ldb + (size_t)kbeg * C::BKB - GROUP_SPAN, (b_rows_ - 1) * p.ldb + kbytes + GROUP_SPAN);
+            const uint32_t chunk = (((lane & 7) - (lane >> 3)) & 7) * 16;          // rotation: see lds_slot
 #pragma unroll
-            for (int i = 0; i < C::LPT; ++i) vo_copy[i] = (i < LPT_A ? voff_a : voff_b) + load_soff(i, 0);
+            for (int i = 0; i < C::LPT; ++i) {
+                const bool is_a = i < LPT_A;
+                const int il = is_a ? i : i - LPT_A;
+                const uint32_t q = wave * (is_a ? LPT_A : LPT_B) + il;
+                const uint32_t row = (q >> 1) * 16 + (q & 1) * 8 + (lane >> 3);
+                vo_copy[i] = row * (is_a ? p.lda : p.ldb) + chunk + GROUP_SPAN - (il & 3) * 1024;
+            }
         }
+        // one LDS-DMA instruction with the immediate offset 1024 * k (a literal: the builtin wants a constant)
+        auto dma = [&](const __amdgpu_buffer_rsrc_t &rs, char *dst, uint32_t vo, uint32_t so, int k) {
+            switch (k) {
+                case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void *)dst, 16, vo, so, 0, 0); break;
+                case 1: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void *)dst, 16, vo, so, 1024, 0); break;
+                case 2: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void *)dst, 16, vo, so, 2048, 0); break;
+                default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void *)dst, 16, vo, so, 3072, 0); break;
+            }
+        };
         auto issue_a1 = [&](int i, int kt, int buf) {
             if constexpr (DBG & 2) return;
-            lds_void *dst = (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024);
-            if constexpr (VOFF_PER_COPY)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, vo_copy[i], (uint32_t)kt * C::BKB, 0, 0);
-            else
+            if constexpr (VOFF_PER_COPY) {
+                char *grp = smem + buf * C::A_BYTES + (wave * LPT_A + (i & ~3)) * 1024;
+                dma(ra_g, grp, vo_copy[i], (uint32_t)kt * C::BKB, i & 3);
+            } else {
+                lds_void *dst = (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, load_soff(i, kt), 0, 0);
+            }
         };
         auto issue_b1 = [&](int i, int kt) {
             if constexpr (DBG & 2) return;
-            lds_void *dst = (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (wave + i * C::NW) * 1024 - C::A_BYTES);
-            if constexpr (VOFF_PER_COPY)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vo_copy[i], (uint32_t)kt * C::BKB, 0, 0);
-            else
+            if constexpr (VOFF_PER_COPY) {
+                const int il = i - LPT_A;
+                char *grp = smem + B_BASE + (kt & 1) * C::B_BYTES + (wave * LPT_B + (il & ~3)) * 1024;
+                dma(rb_g, grp, vo_copy[i], (uint32_t)kt * C::BKB, il & 3);
+            } else {
+                lds_void *dst = (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (wave + i * C::NW) * 1024 - C::A_BYTES);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, load_soff(i, kt), 0, 0);
+            }
         };
         auto next_buf = [&](int bufi) { return bufi + 1 == NA_BUF ? 0 : bufi + 1; };
         if constexpr (C::PIPE == PIPE_SOLO) {
@@ -717,6 +750,21 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());
                 phase_barrier();
                 int kt = 0;
+                if constexpr (PINNED) {
+                    // Six steps at a time (the A ring has three buffers, B two): inside the group the buffer of every
+                    // read and copy is a constant, so the ring arithmetic (two dozen scalar and vector adds per
+                    // step) folds into immediate offsets.  One wave per SIMD: what is not issued is MFMA time.
+                    for (; kt + 6 <= nk; kt += 6) {
+#pragma unroll
+                        for (int j = 0; j < 6; ++j) {
+                            a_rd = j % 3;
+                            a_wr = (j + 2) % 3;
+                            step(kt + j);
+                        }
+                    }
+                    a_rd = 0;            // kt is a multiple of six here
+                    a_wr = 2;
+                }
                 for (; kt < nk; ++kt) step(kt);
                 __builtin_amdgcn_s_waitcnt(0x0070);      // copies landed, reads done, before LDS serves the epilogue
                 phase_barrier();

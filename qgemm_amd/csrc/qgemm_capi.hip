@@ -206,12 +206,13 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
         int vi = choose_by_cost(tab, count, M, N, ksteps, block, cus, may_split, nsplit_out);
         if (vi >= 0) {
             // 256 x 256, int8 and 16-bit types: the 8-wave form needs fewer cycles per tile, the 4-wave form a third
-            // fewer LDS reads.  When the tiles fill whole rounds of CUs the part runs at its power limit and the
-            // 4-wave form wins by 1 % (higher clock); in a partly filled round the clock is not what limits and the
-            // 8-wave form wins by 1 - 6 %.  (fp8 per-matrix: the 4-wave form either way; block scales: 8 waves.)
+            // fewer LDS reads.  With at least one full round of CUs the part runs at its power limit and the 4-wave
+            // form wins by 2 - 3 % (higher clock; level in the partly filled rounds of such shapes); with fewer
+            // tiles than CUs the clock is not what limits and the 8-wave form wins by 1 - 5 %.  (fp8 per-matrix:
+            // the 4-wave form either way; block scales: 8 waves.)
             const Variant &v = tab[vi];
             const size_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
-            if (v.bm == 256 && v.bn == 256 && v.threads == 512 && !block && kmaj == 0 && *nsplit_out <= 1 && tiles % cus == 0)
+            if (v.bm == 256 && v.bn == 256 && v.threads == 512 && !block && kmaj == 0 && *nsplit_out <= 1 && tiles >= (size_t)cus)
                 for (int i = 0; i < count; ++i)
                     if (tab[i].bm == 256 && tab[i].bn == 256 && tab[i].threads == 256 && tab[i].lds_bytes == v.lds_bytes &&
                         !std::strcmp(tab[i].name, "256x256_w2x2_solo"))
@@ -309,7 +310,8 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
         q.M > 128 && q.kmaj == 0) {
         uint32_t ns = 0;
         double t_single = 0;
-        if (choose_by_cost(tab, count, q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, false, &ns, &t_single) == vi) {
+        const int ci = choose_by_cost(tab, count, q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, false, &ns, &t_single);
+        if (ci >= 0 && tab[ci].bm == tab[vi].bm && tab[ci].bn == tab[vi].bn && tab[ci].kgroups == tab[vi].kgroups) {
             const size_t m_main = rows_for_full_rounds(tab, count, tab[vi], q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, t_single);
             if (m_main) {
                 NtProblem q_main = q, q_rest = q;
