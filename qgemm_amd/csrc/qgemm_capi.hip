@@ -135,11 +135,12 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 // everything else goes to the any-shape kernel.
 bool mfma_shape_ok(const NtProblem &q) {
     const size_t es = (q.arith == AR_BF16 || q.arith == AR_F16) ? 2 : 1, krows = q.Kbytes / es;
-    // 32-bit buffer offsets: 256 tile rows of a K-contiguous operand, every k row of a K-major one
+    // 32-bit buffer offsets: 256 tile rows of a K-contiguous operand (plus the 3072 bytes by which the solo kernels
+    // shift their descriptors), every k row of a K-major one
     const bool a_ok = (q.kmaj & 1) ? (krows * q.lda_bytes < ((size_t)1 << 32) && q.lda_bytes >= q.M * es)
-                                   : q.lda_bytes * 256 < ((size_t)1 << 32);
+                                   : q.lda_bytes * 256 + 4096 < ((size_t)1 << 32);
     const bool b_ok = (q.kmaj & 2) ? (krows * q.ldb_bytes < ((size_t)1 << 32) && q.ldb_bytes >= q.N * es)
-                                   : q.ldb_bytes * 256 < ((size_t)1 << 32);
+                                   : q.ldb_bytes * 256 + 4096 < ((size_t)1 << 32);
     return q.Kbytes % 128 == 0 && q.Kbytes > 0 && q.lda_bytes % 16 == 0 && q.ldb_bytes % 16 == 0 && a_ok && b_ok &&
            q.M < ((size_t)1 << 31) && q.N < ((size_t)1 << 31) && q.ldc < ((size_t)1 << 32);
 }
