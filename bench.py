@@ -214,7 +214,13 @@ def main():
         _, ms = _time_launches(lambda: Q.int8_mm(ai, bi, sai, sbi, cf), max(5, args.steps // 2), 3)
         extra["int8_per_matrix_%d" % M] = {"tflops": flops / ms / 1e9, "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["i8"],
                                            "ms": ms, "kernel": Q.last_config()}
-        del ai, bi, cf
+        # the same product with bf16 output (half the bytes of C; what the headline's fp8 run writes)
+        cb16 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        _, ms = _time_launches(lambda: Q.int8_mm(ai, bi, sai, sbi, cb16), max(5, args.steps // 2), 3)
+        extra["int8_per_matrix_%d_bf16_out" % M] = {"tflops": flops / ms / 1e9,
+                                                    "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["i8"], "ms": ms,
+                                                    "kernel": Q.last_config()}
+        del ai, bi, cf, cb16
         # cfg 2: int8 4096^3 -> f32
         m2 = 4096
         ai, sai = _quant_i8(torch.randn(m2, m2, device=dev))
