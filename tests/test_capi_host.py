@@ -112,6 +112,14 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2560, 2560, 2560) == "128x128_w2x2_dma"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x2_solo"
     assert plan(Q.DT_BF16, 0, 0, 512, 4096, 4096) == "64x128_w1x4_k2"
+    # a partly empty last round of 256 x 256 tiles: its rows become a second launch with smaller tiles
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 6144, 6144) == "256x256_w2x2_solo+128x128_w2x2_dma"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 6144, 6144) == "256x256_w2x4_solo8+128x128_w2x2_dma"
+    Q.set_option("row_split", 0)
+    try:
+        assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 6144, 6144) == "256x256_w2x2_solo"
+    finally:
+        Q.set_option("row_split", 1)
     # operands stored K-major: read as stored where that is cheaper than transposing, else transposed first
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 2048, 2048, 2048) == "128x128_w2x2_dma_tn"
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 6144, 4608, 7168) == "transpose+256x256_w2x4_solo8"
