@@ -147,7 +147,7 @@ bool mfma_shape_ok(const NtProblem &q) {
 
 // Which tile, and how many K slices.
 //
-// M > 128: a cost estimate over the tiles worth having there (256 x 256 solo, 128 x 128 in two forms, 64 x 128, 128 x 32) and
+// M > 64: a cost estimate over the tiles worth having there (256 x 256 solo, 128 x 128 in two forms, 64 x 128, 128 x 32) and
 // 1 / 2 / 4 / 8 K slices.  Workgroups run in rounds of CUs x (workgroups that fit a CU); a round costs
 // (K steps x time per step + a fixed prologue / epilogue), a last partial round that leaves a 128 x 128
 // workgroup alone on its CU runs its steps faster, and a K split pays a second launch plus the traffic of the
@@ -157,8 +157,10 @@ bool mfma_shape_ok(const NtProblem &q) {
 // row with two K groups (one per CU: it only wins where there are no more tiles than CUs), 0.45 us for 64 x 128,
 // 0.36 us for 128 x 32.
 //
-// M <= 128 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
-// workgroup, else the shortest tile that covers the rows; narrow tiles instead of a K split.
+// M <= 64 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
+// workgroup, else the shortest tile that covers the rows; narrow tiles instead of a K split.  (65 .. 128 rows go
+// through the estimate as well: it keeps the 128 x 32 tile for the short K of config 5 and prefers a 128 x 128 tile
+// with a K split where K is long, 128 x 8192 x 8192 bf16 38 against 48 us.)
 struct TileModel {
     int bm, bn, per_cu;
     double step_shared, step_alone, fixed;     // microseconds
@@ -203,7 +205,7 @@ int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t kst
 int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
                    bool may_split, uint32_t *nsplit_out) {
     *nsplit_out = 0;                                       // 0: no opinion, plan_nt decides
-    if (M > 128 || kmaj) {
+    if (M > 64 || kmaj) {
         int vi = choose_by_cost(tab, count, M, N, ksteps, block, cus, may_split, nsplit_out);
         if (vi >= 0) {
             // 256 x 256, int8 and 16-bit types: the 8-wave form needs fewer cycles per tile, the 4-wave form a third
