@@ -711,8 +711,17 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                                 } else {
                                     side(b);
                                 }
-                                // B(kt)[b] is dead: its registers take B(kt+1)[b]
-                                if (a == TMs - 1 && h == HALVES - 1) rd_b(kt + 1, b);
+                                // B(kt)[b] is dead: its registers take B(kt+1)[b] (where a tile takes two MFMAs:
+                                // each half as soon as its MFMA of the last row is out, so the first halves, which
+                                // the next step needs first, are read half a row earlier)
+                                if constexpr (HALVES == 2) {
+                                    if (a == TMs - 1 && !(DBG & 4)) {
+                                        const char *sb_ = smem + B_BASE + ((kt + 1) & 1) * C::B_BYTES - C::A_BYTES;
+                                        fbr[b][h] = frag_b(sb_, b, h);
+                                    }
+                                } else {
+                                    if (a == TMs - 1) rd_b(kt + 1, b);
+                                }
                             }
                         }
                     }
