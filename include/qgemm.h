@@ -62,8 +62,8 @@ typedef enum qgemm_layout {
 
 /* Library set-up.  Replaces blas::blas_init / blas::blas_destroy
  * (include/blas.h:33-48): selects the current HIP device, loads the kernels.
- * Idempotent; the compute entries call it lazily.  qgemm_shutdown frees the
- * per-device workspace. */
+ * Idempotent; the compute entries call it lazily.  qgemm_shutdown waits for
+ * the device and frees every workspace block. */
 int qgemm_init(void);
 int qgemm_shutdown(void);
 
@@ -100,6 +100,19 @@ int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const void *A, size_t 
 int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
                       const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N,
                       size_t K, int split_k, void *stream);
+
+/* Library workspace (no reference counterpart: the reference's entries take none).  Calls that split K, that
+ * take operands or scales in an arrangement the kernels do not read directly, and the per-matrix quantiser keep
+ * their intermediate data in one device block owned by the library and grown on demand.  A block that is
+ * outgrown is replaced but stays allocated until qgemm_shutdown, so launches already enqueued and graphs
+ * already captured remain valid.  Calls on different streams share the block: each such call waits (on the
+ * device, through an event) for the previous user on another stream.  While a stream is being captured into a
+ * graph the library neither allocates nor touches that event: a call that would have to grow the block returns
+ * QGEMM_ERR_ALLOC, and replays of graphs that use the workspace must not overlap other users of it.
+ * qgemm_reserve_workspace makes the block at least `bytes` large ahead of time; qgemm_workspace_info reports
+ * its address and size (NULL / 0 before first use). */
+int qgemm_reserve_workspace(size_t bytes);
+int qgemm_workspace_info(void **base, size_t *bytes);
 
 /* out[n*M + m] = in[m*N + n] for 1-, 2- or 4-byte elements.
  * Replaces matrix_transpose<T> (src/transpose/transpose.cu:60-74), which

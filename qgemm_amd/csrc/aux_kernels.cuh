@@ -80,7 +80,8 @@ __global__ void __launch_bounds__(256) gemm_strided_kernel(const StridedArgs p) 
                 part += load_elem<IN_DT>(p.A, (size_t)m * p.a_rs + k * p.a_cs) *
                         load_elem<IN_DT>(p.B, (size_t)n * p.b_ns + k * p.b_ks);
             const uint32_t kb = k0 / kScaleBlock;
-            acc += (part * p.as[m * p.as_ms + kb * p.as_ks]) * p.bs[(n / kScaleBlock) * p.bs_ns + kb * p.bs_ks];
+            acc += (part * p.as[(size_t)m * p.as_ms + (size_t)kb * p.as_ks]) *
+                   p.bs[(size_t)(n / kScaleBlock) * p.bs_ns + (size_t)kb * p.bs_ks];
         }
         store_out(p.C, idx, acc, p.out_dtype);
         return;

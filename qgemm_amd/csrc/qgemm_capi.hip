@@ -23,17 +23,30 @@ using namespace qgemm;
 
 namespace {
 
+struct WsBlock {
+    void *p = nullptr;
+    size_t bytes = 0;
+};
+
 struct Context {
     std::mutex mu;
     bool ready = false;
     int device = -1;
     int num_cus = 256;
-    void *workspace = nullptr;
-    size_t workspace_bytes = 0;
+    // Workspace (split-K partial planes, transposed operands and scales, quantiser partials): one block for
+    // the process.  A block that is outgrown is replaced and kept in `retired` until qgemm_shutdown: launches
+    // already enqueued and graphs already captured keep pointing at live memory.  Calls on different streams
+    // share the block and are ordered through ws_event: every call that used the workspace records it on its
+    // stream when it has enqueued its launches, and a call on another stream waits for it first.
+    WsBlock ws;
+    std::vector<void *> retired;
+    hipEvent_t ws_event = nullptr;
+    hipStream_t ws_last_stream = nullptr;
+    bool ws_event_recorded = false;
+    bool ws_used_by_call = false;              // the running entry asked for the workspace
     long force_config = -1;     // index into the variant table, -1 = heuristic
     long force_split = 0;       // 0 = heuristic
     long force_group_m = 0;     // 0 = default
-    long debug_flags = 0;       // GemmArgs::debug
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes
     std::string last_config;
@@ -64,26 +77,65 @@ int ensure_init_locked() {
     return QGEMM_OK;
 }
 
-// Grows the per-process workspace (split-K partial planes, transposed operands).
-// Calls that use it are ordered by the stream they are enqueued on; concurrent
-// calls on different streams would share it and must not overlap.
-int ensure_workspace_locked(size_t bytes, void **out) {
-    if (bytes > g_ctx.workspace_bytes) {
-        if (g_ctx.workspace) {
-            HIP_TRY(hipDeviceSynchronize());
-            HIP_TRY(hipFree(g_ctx.workspace));
-            g_ctx.workspace = nullptr;
-            g_ctx.workspace_bytes = 0;
-        }
-        size_t want = std::max(bytes, (size_t)64 << 20);
-        void *p = nullptr;
-        if (hipMalloc(&p, want) != hipSuccess) return QGEMM_ERR_ALLOC;
-        g_ctx.workspace = p;
-        g_ctx.workspace_bytes = want;
+bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
     }
-    *out = g_ctx.workspace;
+    return cap != hipStreamCaptureStatusNone;
+}
+
+// Workspace of `bytes` for a call enqueued on `stream`.
+// The library's block, grown when too small.  Growing allocates a new block and retires the old
+//     one without freeing it (see Context).  While the stream is being captured into a graph nothing is
+//     allocated and no event is waited for or recorded: a call that would have to grow the block fails with
+//     QGEMM_ERR_ALLOC (the caller reserves the room before the capture, qgemm_reserve_workspace, or runs the
+//     call once eagerly), and ordering replays against other users of the workspace is the caller's business.
+int ensure_workspace_locked(size_t bytes, hipStream_t stream, void **out) {
+    const bool capturing = stream_is_capturing(stream);
+    if (bytes > g_ctx.ws.bytes) {
+        if (capturing) return QGEMM_ERR_ALLOC;
+        const size_t want = std::max({bytes, 2 * g_ctx.ws.bytes, (size_t)64 << 20});
+        void *p = nullptr;
+        if (hipMalloc(&p, want) != hipSuccess) {
+            (void)hipGetLastError();
+            return QGEMM_ERR_ALLOC;
+        }
+        if (g_ctx.ws.p) g_ctx.retired.push_back(g_ctx.ws.p);
+        g_ctx.ws.p = p;
+        g_ctx.ws.bytes = want;
+    }
+    if (!capturing) {
+        if (g_ctx.ws_event_recorded && g_ctx.ws_last_stream != stream && !g_ctx.ws_used_by_call)
+            HIP_TRY(hipStreamWaitEvent(stream, g_ctx.ws_event, 0));
+        g_ctx.ws_used_by_call = true;
+    }
+    *out = g_ctx.ws.p;
     return QGEMM_OK;
 }
+
+// Around the body of every entry that may use the workspace: when it did, the end of its launches is recorded
+// on its stream for the next user on another stream to wait for.
+struct WorkspaceUse {
+    hipStream_t stream;
+    explicit WorkspaceUse(hipStream_t s) : stream(s) { g_ctx.ws_used_by_call = false; }
+    ~WorkspaceUse() {
+        if (!g_ctx.ws_used_by_call) return;
+        g_ctx.ws_used_by_call = false;
+        if (!g_ctx.ws_event && hipEventCreateWithFlags(&g_ctx.ws_event, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            g_ctx.ws_event = nullptr;
+            return;
+        }
+        if (hipEventRecord(g_ctx.ws_event, stream) == hipSuccess) {
+            g_ctx.ws_event_recorded = true;
+            g_ctx.ws_last_stream = stream;
+        } else {
+            (void)hipGetLastError();
+        }
+    }
+};
 
 // kmaj: GemmCfg::KMAJ of the wanted family (0: both operands K-contiguous)
 const Variant *table_for(int arith, bool block, int kmaj, int *count) {
@@ -141,7 +193,9 @@ bool mfma_shape_ok(const NtProblem &q) {
                                    : q.lda_bytes * 256 + 4096 < ((size_t)1 << 32);
     const bool b_ok = (q.kmaj & 2) ? (krows * q.ldb_bytes < ((size_t)1 << 32) && q.ldb_bytes >= q.N * es)
                                    : q.ldb_bytes * 256 + 4096 < ((size_t)1 << 32);
-    return q.Kbytes % 128 == 0 && q.Kbytes > 0 && q.lda_bytes % 16 == 0 && q.ldb_bytes % 16 == 0 && a_ok && b_ok &&
+    // block scales: the kernel addresses a_scale with 32-bit byte offsets ((kb * as_ks + m) * 4)
+    const bool s_ok = !q.block || ((q.Kbytes + 127) / 128) * std::max<size_t>(q.M, q.as_ks) * 4 < ((size_t)1 << 32);
+    return q.Kbytes % 128 == 0 && q.Kbytes > 0 && q.lda_bytes % 16 == 0 && q.ldb_bytes % 16 == 0 && a_ok && b_ok && s_ok &&
            q.M < ((size_t)1 << 31) && q.N < ((size_t)1 << 31) && q.ldc < ((size_t)1 << 32);
 }
 
@@ -486,7 +540,7 @@ int launch_nt(NtProblem q, hipStream_t stream) {
     void *ws = nullptr;
     const size_t split_room = (pl.split_bytes + 255) / 256 * 256, as_room = scales_room(q);
     if (split_room + as_room) {
-        st = ensure_workspace_locked(split_room + as_room, &ws);
+        st = ensure_workspace_locked(split_room + as_room, stream, &ws);
         if (st != QGEMM_OK) return st;
     }
     if (as_room) {
@@ -505,6 +559,7 @@ int launch_strided_t(const StridedArgs &s, hipStream_t stream) {
 
 int launch_strided(int in_dtype, const StridedArgs &s, hipStream_t stream) {
     g_ctx.last_config = "strided_any_shape";
+    if ((s.N + 15) / 16 > 0x7FFFFFFFu || (s.M + 15) / 16 > 65535u) return QGEMM_ERR_TOO_LARGE;    // grid limits
     switch (in_dtype) {
         case QGEMM_DT_I8: return launch_strided_t<QGEMM_DT_I8>(s, stream);
         case QGEMM_DT_F8E4M3: return launch_strided_t<QGEMM_DT_F8E4M3>(s, stream);
@@ -556,7 +611,7 @@ int quantize_t(int mode, QuantArgs &a, hipStream_t stream) {
         // two passes: partial maxima (one per workgroup) into the workspace, then scale and cast
         const uint32_t nblk = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(2048, (groups + 1023) / 1024));
         void *ws = nullptr;
-        int st = ensure_workspace_locked(nblk * sizeof(float), &ws);
+        int st = ensure_workspace_locked(nblk * sizeof(float), stream, &ws);
         if (st != QGEMM_OK) return st;
         a.partial = (float *)ws;
         a.npartial = nblk;
@@ -593,12 +648,16 @@ QGEMM_EXPORT int qgemm_init(void) {
 
 QGEMM_EXPORT int qgemm_shutdown(void) {
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    if (g_ctx.workspace) {
+    if (g_ctx.ws.p || !g_ctx.retired.empty()) {
         (void)hipDeviceSynchronize();
-        (void)hipFree(g_ctx.workspace);
+        if (g_ctx.ws.p) (void)hipFree(g_ctx.ws.p);
+        for (void *p : g_ctx.retired) (void)hipFree(p);
     }
-    g_ctx.workspace = nullptr;
-    g_ctx.workspace_bytes = 0;
+    if (g_ctx.ws_event) (void)hipEventDestroy(g_ctx.ws_event);
+    g_ctx.ws = WsBlock();
+    g_ctx.retired.clear();
+    g_ctx.ws_event = nullptr;
+    g_ctx.ws_event_recorded = false;
     g_ctx.ready = false;
     return QGEMM_OK;
 }
@@ -633,7 +692,6 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     if (!std::strcmp(key, "force_config")) g_ctx.force_config = value;
     else if (!std::strcmp(key, "force_split")) g_ctx.force_split = value;
     else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
-    else if (!std::strcmp(key, "debug_flags")) g_ctx.debug_flags = value;
     else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
     else if (!std::strcmp(key, "row_split")) g_ctx.row_split = value;
     else return QGEMM_ERR_INVALID_ARG;
@@ -709,6 +767,7 @@ QGEMM_EXPORT int qgemm_quantize(int in_dtype, int out_dtype, int mode, const voi
     int st = ensure_init_locked();
     if (st != QGEMM_OK) return st;
     hipStream_t stream = (hipStream_t)stream_;
+    WorkspaceUse ws_use(stream);
     QuantArgs a;
     std::memset(&a, 0, sizeof(a));
     a.x = x;
@@ -741,6 +800,7 @@ QGEMM_EXPORT int qgemm_transpose(int elem_bytes, const void *in, void *out, size
     if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) return QGEMM_ERR_UNSUPPORTED;
     if (M == 0 || N == 0) return QGEMM_OK;
     if (!in || !out) return QGEMM_ERR_INVALID_ARG;
+    if (M >= ((size_t)1 << 31) || N >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     int st = ensure_init_locked();
     if (st != QGEMM_OK) return st;
@@ -759,6 +819,7 @@ QGEMM_EXPORT int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const voi
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     int st = ensure_init_locked();
     if (st != QGEMM_OK) return st;
+    WorkspaceUse ws_use(stream);
 
     const size_t eb = dtype_bytes(in_dtype);
     NtProblem q;
@@ -796,7 +857,7 @@ QGEMM_EXPORT int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const voi
             if (st != QGEMM_OK) return st;
             const size_t split_room = (pl.split_bytes + 255) / 256 * 256;
             void *ws = nullptr;
-            st = ensure_workspace_locked(split_room + N * K * eb, &ws);
+            st = ensure_workspace_locked(split_room + N * K * eb, stream, &ws);
             if (st != QGEMM_OK) return st;
             void *bt = (char *)ws + split_room;
             st = launch_transpose((int)eb, B, bt, K, N, stream);
@@ -806,6 +867,7 @@ QGEMM_EXPORT int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const voi
         }
     }
 
+    if (M >= ((size_t)1 << 32) || N >= ((size_t)1 << 32) || K >= ((size_t)1 << 32)) return QGEMM_ERR_TOO_LARGE;
     StridedArgs s;
     std::memset(&s, 0, sizeof(s));
     s.A = A;
@@ -829,7 +891,11 @@ QGEMM_EXPORT int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const voi
     return launch_strided(in_dtype, s, stream);
 }
 
-QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
+}  // extern "C"
+
+namespace {
+
+int scaled_gemm_entry(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
                       const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N, size_t K,
                       int split_k, void *stream_) {
     if (in_dtype != QGEMM_DT_I8 && in_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
@@ -852,6 +918,7 @@ QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, 
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     int st = ensure_init_locked();
     if (st != QGEMM_OK) return st;
+    WorkspaceUse ws_use(stream);
 
     const bool block = scale_mode == QGEMM_SCALE_BLOCK128;
     const uint32_t KB = (uint32_t)((K + 127) / 128), NBLK = (uint32_t)((N + 127) / 128);
@@ -900,7 +967,7 @@ QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, 
         const size_t split_room = (pl.split_bytes + 255) / 256 * 256;
         const size_t at_bytes = (M * K + 255) / 256 * 256;
         void *ws = nullptr;
-        st = ensure_workspace_locked(split_room + at_bytes + N * K, &ws);
+        st = ensure_workspace_locked(split_room + at_bytes + N * K, stream, &ws);
         if (st != QGEMM_OK) return st;
         char *at = (char *)ws + split_room, *bt = at + at_bytes;
         // M, N, K are multiples of 32 here: both matrices qualify for the register-permute byte transpose
@@ -927,6 +994,7 @@ QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, 
         return run_nt(q, pl, ws, stream);
     }
 
+    if (M >= ((size_t)1 << 32) || N >= ((size_t)1 << 32) || K >= ((size_t)1 << 32)) return QGEMM_ERR_TOO_LARGE;
     StridedArgs s;
     std::memset(&s, 0, sizeof(s));
     s.A = A;
@@ -949,6 +1017,41 @@ QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, 
     s.out_dtype = out_dtype;
     s.scale_mode = raw_acc ? 0 : scale_mode;
     return launch_strided(in_dtype, s, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
+                      const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N, size_t K,
+                      int split_k, void *stream) {
+    return scaled_gemm_entry(in_dtype, out_dtype, scale_mode, layout, A, B, a_scale, b_scale, C, ldC, M, N, K, split_k,
+                             stream);
+}
+
+QGEMM_EXPORT int qgemm_reserve_workspace(size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    int st = ensure_init_locked();
+    if (st != QGEMM_OK) return st;
+    if (bytes <= g_ctx.ws.bytes) return QGEMM_OK;
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return QGEMM_ERR_ALLOC;
+    }
+    if (g_ctx.ws.p) g_ctx.retired.push_back(g_ctx.ws.p);
+    g_ctx.ws.p = p;
+    g_ctx.ws.bytes = bytes;
+    return QGEMM_OK;
+}
+
+QGEMM_EXPORT int qgemm_workspace_info(void **base, size_t *bytes) {
+    if (!base || !bytes) return QGEMM_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    *base = g_ctx.ws.p;
+    *bytes = g_ctx.ws.bytes;
+    return QGEMM_OK;
 }
 
 // ---------------------------------------------------------------------------
@@ -1043,6 +1146,9 @@ QGEMM_EXPORT int qgemm_selftest_layouts(char *buf, size_t buflen) {
                     std::snprintf(line, sizeof(line), "lds_dma: soffset %s part of the buffer range check\n",
                                   z ? "IS" : "is NOT");
                     rep += line;
+                    // tile rows past M or N are kept out of reach by the range check alone (the row block of a
+                    // copy sits in the scalar offset in the simple and ping-pong pipelines)
+                    if (!z) all_ok = false;
                     continue;
                 }
                 if (off + 16 > (uint64_t)nsrc) {

@@ -36,14 +36,29 @@ void need_device(const torch::Tensor &t, const char *name) {
     if (!t.is_cuda()) throw std::runtime_error(std::string("qgemm_python: ") + name + " must be a device tensor");
 }
 
+// The kernels decode OCP e4m3 (torch.float8_e4m3fn or raw codes as uint8); the gfx942 "fnuz" encoding has another
+// bias and another NaN and is refused.
+void need_fp8(const torch::Tensor &t, const char *name) {
+    if (t.scalar_type() != torch::kFloat8_e4m3fn && t.scalar_type() != torch::kUInt8)
+        throw std::runtime_error(std::string("qgemm_python: ") + name + " must be float8_e4m3fn (OCP e4m3) or uint8 codes");
+}
+
+// c is [m, n] with unit inner stride; its row stride becomes ldC
+void need_out(const torch::Tensor &c, size_t m, size_t n) {
+    if (c.dim() != 2 || (size_t)c.size(0) != m || (size_t)c.size(1) != n || c.stride(1) != 1 || (m > 1 && (size_t)c.stride(0) < n))
+        throw std::runtime_error("qgemm_python: c must be [m, n] with unit inner stride");
+}
+
 // The reference's contract (hip_mix_gemm_kernel.cpp:425-439): a is [m, k] column-major (storage a[i + j*m]),
 // b is [n, k] column-major (storage [k, n] row-major), a_scale [m, k/128] and b_scale [n/128, k/128]
 // column-major, c [m, n] row-major bf16; m = a.size(0), n = b.size(0), k = a.size(1).
 void fp8_mm(torch::Tensor a, torch::Tensor b, torch::Tensor as, torch::Tensor bs, torch::Tensor c) {
     need_device(a, "a"); need_device(b, "b"); need_device(as, "a_scale"); need_device(bs, "b_scale"); need_device(c, "c");
     const size_t m = a.size(0), n = b.size(0), k = a.size(1);
+    need_fp8(a, "a"); need_fp8(b, "b");
+    need_out(c, m, n);
     check(qgemm_scaled_gemm(QGEMM_DT_F8E4M3, dtype_of(c), QGEMM_SCALE_BLOCK128, QGEMM_LAYOUT_REFERENCE, a.data_ptr(),
-                            b.data_ptr(), as.data_ptr<float>(), bs.data_ptr<float>(), c.data_ptr(), n, m, n, k, 0,
+                            b.data_ptr(), as.data_ptr<float>(), bs.data_ptr<float>(), c.data_ptr(), c.stride(0), m, n, k, 0,
                             current_stream()),
           "fp8_mm");
 }
@@ -55,15 +70,19 @@ void scaled_mm(torch::Tensor a, torch::Tensor b, torch::Tensor as, torch::Tensor
     if (!a.is_contiguous() || !b.is_contiguous() || a.size(1) != b.size(1))
         throw std::runtime_error(std::string(what) + ": a [m, k] and b [n, k] must be contiguous with equal k");
     const size_t m = a.size(0), n = b.size(0), k = a.size(1);
+    need_out(c, m, n);
     check(qgemm_scaled_gemm(dtype_of(a), dtype_of(c), QGEMM_SCALE_PER_MATRIX, QGEMM_LAYOUT_K_CONTIGUOUS, a.data_ptr(),
                             b.data_ptr(), as.data_ptr<float>(), bs.data_ptr<float>(), c.data_ptr(), c.stride(0), m, n, k, 0,
                             current_stream()),
           what);
 }
 void int8_mm(torch::Tensor a, torch::Tensor b, torch::Tensor as, torch::Tensor bs, torch::Tensor c) {
+    if (a.scalar_type() != torch::kInt8 || b.scalar_type() != torch::kInt8)
+        throw std::runtime_error("qgemm_python: int8_mm takes int8 operands");
     scaled_mm(a, b, as, bs, c, "int8_mm");
 }
 void fp8_mm_per_matrix(torch::Tensor a, torch::Tensor b, torch::Tensor as, torch::Tensor bs, torch::Tensor c) {
+    need_fp8(a, "a"); need_fp8(b, "b");
     scaled_mm(a, b, as, bs, c, "fp8_mm_per_matrix");
 }
 
@@ -72,6 +91,7 @@ void bf16_mm(torch::Tensor a, torch::Tensor b, torch::Tensor c) {
     need_device(a, "a"); need_device(b, "b"); need_device(c, "c");
     if (a.size(1) != b.size(1) || a.stride(1) != 1 || b.stride(1) != 1 || c.stride(1) != 1)
         throw std::runtime_error("bf16_mm: a [m, k] and b [n, k] with unit inner strides");
+    need_out(c, a.size(0), b.size(0));
     check(qgemm_gemm(dtype_of(a), dtype_of(c), QGEMM_B_NK, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), c.data_ptr(),
                      c.stride(0), a.size(0), b.size(0), a.size(1), current_stream()),
           "bf16_mm");

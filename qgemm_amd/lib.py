@@ -37,6 +37,8 @@ SIGNATURES = {
     "qgemm_status_string": (C.c_char_p, [_i]),
     "qgemm_gemm": (_i, [_i, _i, _i, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp]),
     "qgemm_scaled_gemm": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _i, _vp]),
+    "qgemm_reserve_workspace": (_i, [_sz]),
+    "qgemm_workspace_info": (_i, [C.POINTER(_vp), C.POINTER(_sz)]),
     "qgemm_transpose": (_i, [_i, _vp, _vp, _sz, _sz, _vp]),
     "qgemm_quantize": (_i, [_i, _i, _i, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _sz, _sz, _vp]),
     "qgemm_tile_map": (_i, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32),

@@ -103,6 +103,20 @@ def scaled_gemm(A, B, a_scale, b_scale, C_out, M, N, K, scale_mode, layout=LAYOU
     return C_out
 
 
+def _need_fp8(*ts):
+    """The kernels decode OCP e4m3 (torch.float8_e4m3fn, or its raw codes as uint8).  The gfx942 "fnuz" encoding
+    the reference's fp8_mm names has another bias and another NaN: refuse it rather than compute with every value
+    doubled."""
+    for t in ts:
+        if t.dtype not in (torch.float8_e4m3fn, torch.uint8):
+            raise TypeError(f"fp8 operands must be torch.float8_e4m3fn (OCP e4m3) or uint8 codes, got {t.dtype}")
+
+
+def _need_out(c, m, n):
+    if c.dim() != 2 or tuple(c.shape) != (m, n) or c.stride(1) != 1 or (m > 1 and c.stride(0) < n):
+        raise ValueError(f"c must be [{m}, {n}] with unit inner stride, got shape {tuple(c.shape)} strides {c.stride()}")
+
+
 def fp8_mm(a, b, a_scale, b_scale, c):
     """The reference entry (hip_mix_gemm_kernel.cpp:425-439, 508-516):
       a        [m, k] fp8, column-major  (storage a[i + j*m])
@@ -111,8 +125,10 @@ def fp8_mm(a, b, a_scale, b_scale, c):
       c        [m, n] bf16, row-major
     m = a.size(0), n = b.size(0), k = a.size(1) exactly as the reference reads them."""
     m, n, k = a.size(0), b.size(0), a.size(1)
+    _need_fp8(a, b)
+    _need_out(c, m, n)
     return scaled_gemm(a, b, a_scale, b_scale, c, m, n, k, SCALE_BLOCK128, LAYOUT_REFERENCE, in_dtype=DT_F8E4M3,
-                       ldC=n)
+                       ldC=c.stride(0))
 
 
 def int8_mm(a, b, a_scale, b_scale, c, split_k=0):
@@ -120,7 +136,11 @@ def int8_mm(a, b, a_scale, b_scale, c, split_k=0):
     c [m,n] fp32 / bf16 / fp16, or int32 for the raw accumulators."""
     m, k = a.shape
     n = b.shape[0]
-    return scaled_gemm(a, b, a_scale, b_scale, c, m, n, k, SCALE_PER_MATRIX, split_k=split_k, in_dtype=DT_I8)
+    if a.dtype != torch.int8 or b.dtype != torch.int8:
+        raise TypeError(f"int8_mm takes int8 operands, got {a.dtype} and {b.dtype}")
+    _need_out(c, m, n)
+    return scaled_gemm(a, b, a_scale, b_scale, c, m, n, k, SCALE_PER_MATRIX, split_k=split_k, in_dtype=DT_I8,
+                       ldC=c.stride(0))
 
 
 def bf16_mm(a, b, c):

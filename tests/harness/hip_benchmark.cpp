@@ -139,8 +139,9 @@ static void bench_bf16(const Shape &s, int warmup, int runs, double tol) {
     for (const Row &r : rows) {
         HIP_OK(hipMemset(dC, 0, M * N * 4));
         const __hip_bfloat16 *b = r.b_is_nk ? dBt : dB;
-        const size_t ldB = r.b_is_nk ? K : N;
-        const double ms = time_launches([&] { r.fn(dA, K, b, ldB, dC, N, M, N, K); }, warmup, runs);
+        // every entry is called with ldA = K, ldB = N, ldC = N, the N x K ones included, as the reference's
+        // harness does (tests/includes/test_config.h:238): the entries index dense operands and ignore ldA / ldB
+        const double ms = time_launches([&] { r.fn(dA, K, b, N, dC, N, M, N, K); }, warmup, runs);
         HIP_OK(hipMemcpy(got.data(), dC, M * N * 4, hipMemcpyDeviceToHost));
         double max_err = 0;
         for (size_t i = 0; i < M * N; ++i) max_err = std::max(max_err, std::fabs((double)got[i] - (double)ref[i]));

@@ -155,3 +155,81 @@ def test_c_abi_header_is_plain_c(tmp_path):
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"),
                     "-c", str(src), "-o", str(tmp_path / "use.o")], check=True)
+
+
+def test_too_large_is_reported_not_wrapped():
+    """Dimensions beyond what the kernels index come back as QGEMM_ERR_TOO_LARGE (9) instead of wrapping around:
+    more tiles than a grid holds (plan_nt), a transpose side of 2^31, block scales past 32-bit byte offsets."""
+    lib = L.load_library()
+    one = C.c_void_p(16)
+    with pytest.raises(Q.QgemmError) as e:
+        Q.plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 1 << 22, 1 << 22, 128)
+    assert e.value.status == 9
+    assert lib.qgemm_transpose(2, one, one, 1 << 31, 4, None) == 9
+    assert lib.qgemm_transpose(1, one, one, 4, 1 << 31, None) == 9
+    # block scales: M * ceil(K / 128) * 4 bytes >= 2^32 cannot go to the MFMA kernel
+    assert Q.plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 1 << 20, 256, 1 << 17) == "strided_any_shape"
+
+
+def test_workspace_entries_need_no_device_to_answer():
+    lib = L.load_library()
+    base, size = C.c_void_p(123), C.c_size_t(7)
+    assert lib.qgemm_workspace_info(C.byref(base), C.byref(size)) == 0
+    if lib.qgemm_device_count() == 0:
+        assert base.value is None and size.value == 0
+        assert lib.qgemm_reserve_workspace(1 << 20) == 3          # QGEMM_ERR_NO_DEVICE
+    assert lib.qgemm_workspace_info(None, None) == 1
+
+
+def test_nt_forwarders_pass_dense_strides_like_the_reference(tmp_path):
+    """GEMM_kernel_v3_1 / v4_1 (and the NN entries) ignore the caller's ldA / ldB exactly as the reference's
+    launchers do (sm80_gemm_kernel_v3.1.cu:292 passes K for ldB; tests/includes/test_config.h:238 calls every
+    entry with ldB = N): built against a stub qgemm_gemm that prints what it receives."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    src = tmp_path / "fwd.cpp"
+    src.write_text(r'''
+#include <cstdio>
+#include "gemm.h"
+extern "C" int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const void *, size_t ldA, const void *, size_t ldB,
+                          void *, size_t ldC, size_t M, size_t N, size_t K, void *) {
+    std::printf("%d %d %d %zu %zu %zu %zu %zu %zu\n", in_dtype, out_dtype, layout_b, ldA, ldB, ldC, M, N, K);
+    return 0;
+}
+extern "C" const char *qgemm_status_string(int) { return ""; }
+int main() {
+    const __hip_bfloat16 *a = nullptr, *b = nullptr;
+    float *c = nullptr;
+    GEMM_kernel_v3_1<__hip_bfloat16, float>(a, 64, b, 48, c, 56, 32, 48, 64);   // M=32 N=48 K=64, ldB = N as the harness
+    GEMM_kernel_v4_1<__hip_bfloat16, float>(a, 999, b, 999, c, 48, 32, 48, 64);
+    GEMM_kernel_v3<__hip_bfloat16, float>(a, 999, b, 999, c, 48, 32, 48, 64);
+    return 0;
+}
+''')
+    exe = tmp_path / "fwd"
+    subprocess.run([hipcc, "-std=c++17", "--offload-arch=gfx950", "-I", os.path.join(ROOT, "include"), str(src), "-o",
+                    str(exe)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split("\n")
+    assert out[0] == "1 0 1 64 64 56 32 48 64"      # bf16 -> f32, B is N x K: ldB = K whatever the caller said; ldC kept
+    assert out[1] == "1 0 1 64 64 48 32 48 64"
+    assert out[2] == "1 0 0 64 48 48 32 48 64"      # B is K x N: ldB = N
+
+
+def test_fnuz_fp8_is_refused_not_misread():
+    """torch.float8_e4m3fnuz (the gfx942 encoding the reference's fp8_mm names) has another bias and another NaN
+    code: the wrappers refuse it instead of decoding it as OCP e4m3."""
+    import torch
+    if not hasattr(torch, "float8_e4m3fnuz"):
+        pytest.skip("this torch has no fnuz dtype")
+    a = torch.zeros((32, 128), dtype=torch.uint8).view(torch.float8_e4m3fnuz)
+    s = torch.ones(1)
+    with pytest.raises(TypeError):
+        Q.fp8_mm(a, a, s, s, torch.zeros((32, 32), dtype=torch.bfloat16))
+    ok = torch.zeros((32, 128), dtype=torch.uint8).view(torch.float8_e4m3fn)
+    with pytest.raises(ValueError):          # c with the wrong shape
+        Q.fp8_mm(ok, ok, s, s, torch.zeros((32, 16), dtype=torch.bfloat16))
+    with pytest.raises(ValueError):          # c with a non-unit inner stride
+        Q.fp8_mm(ok, ok, s, s, torch.zeros((32, 64), dtype=torch.bfloat16)[:, ::2])

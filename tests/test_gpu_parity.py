@@ -33,6 +33,8 @@ def test_selftest_layouts():
     ok, report = Q.selftest_layouts()
     print(report, flush=True)
     assert ok, report
+    # tile rows past M / N are kept out of reach by the buffer range check, scalar offset included
+    assert "soffset IS part of the buffer range check" in report
 
 
 # ----------------------------------------------------------------- int8
@@ -148,21 +150,25 @@ def test_fp8_block_scaled_every_variant(variant):
     assert_close(host(c), ref, what=Q.last_config())
 
 
-def test_fp8_block_scaled_power_of_two_scales_bit_exact():
+@pytest.mark.parametrize("variant", [-1] + list(range(N_VARIANTS)))
+@pytest.mark.parametrize("shape", [(64, 256, 512), (272, 392, 768)])
+def test_fp8_block_scaled_power_of_two_scales_bit_exact(variant, shape):
     """Power-of-two scales commute exactly with fp32 arithmetic, and small-integer products sum exactly:
-    the scaled result must equal the oracle bit for bit (catches a wrong scale index)."""
-    M, N, K = 64, 256, 512
-    say("fp8 block pow2")
-    rng = np.random.default_rng(6)
+    the scaled result must equal the oracle bit for bit, in every tile variant and pipeline (a wrong scale
+    index, row or K block, cannot hide behind a tolerance).  Ragged M and N in the second shape."""
+    M, N, K = shape
+    say("fp8 block pow2", shape, "variant", variant)
+    Q.set_option("force_config", variant)
+    rng = np.random.default_rng(6 + variant)
     a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
     b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
     as_ = (2.0 ** rng.integers(-3, 4, size=(M, K // 128))).astype(np.float32)
-    bs = (2.0 ** rng.integers(-3, 4, size=(N // 128, K // 128))).astype(np.float32)
+    bs = (2.0 ** rng.integers(-3, 4, size=((N + 127) // 128, K // 128))).astype(np.float32)
     ref = R.gemm_fp8_block(a, b, as_, bs)
     c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K,
-                  Q.SCALE_BLOCK128)
-    assert np.array_equal(host(c), ref)
+                  Q.SCALE_BLOCK128, split_k=1 if variant >= 0 else 0)
+    assert np.array_equal(host(c), ref), Q.last_config()
 
 
 def test_fp8_mm_reference_layout():
