@@ -71,10 +71,9 @@ def test_no_allocation_during_capture():
     QGEMM_ERR_ALLOC (5) and leaves the block alone."""
     say("workspace growth refused during capture")
     base0, size0 = _info()
-    M, N, K = 4096, 4096, 1024                       # 4 planes of 64 MiB
-    need = M * N * 4 * 4
-    if size0 >= need:
-        pytest.skip("workspace already larger than this test's request")
+    M, N = 4096, 4096                                # planes of 64 MiB: as many as it takes to outgrow the block
+    nsplit = size0 // (M * N * 4) + 2
+    K = 128 * 4 * nsplit
     a = torch.zeros((M, K), dtype=torch.int8, device="cuda")
     b = torch.zeros((N, K), dtype=torch.int8, device="cuda")
     c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
@@ -83,7 +82,7 @@ def test_no_allocation_during_capture():
     status = []
     with torch.cuda.graph(g):
         try:
-            Q.int8_mm(a, b, s, s, c, split_k=4)
+            Q.int8_mm(a, b, s, s, c, split_k=nsplit)
             status.append(0)
         except Q.QgemmError as e:
             status.append(e.status)
