@@ -28,7 +28,8 @@ typedef enum qgemm_status {
     QGEMM_ERR_NOT_DIVISIBLE_M = 6, /* reference dispatch contract: M % 32 != 0       */
     QGEMM_ERR_NOT_DIVISIBLE_N = 7, /*                              N % 32 != 0       */
     QGEMM_ERR_NOT_DIVISIBLE_K = 8, /*                              K % 32 != 0       */
-    QGEMM_ERR_TOO_LARGE = 9      /* a dimension or stride exceeds what kernels index */
+    QGEMM_ERR_TOO_LARGE = 9,     /* a dimension or stride exceeds what kernels index */
+    QGEMM_ERR_SCRATCH_TOO_SMALL = 10 /* qgemm_scaled_gemm_static: the call needs more than the static scratch */
 } qgemm_status_t;
 
 typedef enum qgemm_dtype {
@@ -100,6 +101,19 @@ int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const void *A, size_t 
 int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
                       const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N,
                       size_t K, int split_k, void *stream);
+
+/* qgemm_scaled_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and
+ * same results as qgemm_scaled_gemm; whatever that entry would take from the library workspace (split-K partial
+ * planes, the transposed a_scale of QGEMM_LAYOUT_K_CONTIGUOUS block scales, the transposed operands of
+ * QGEMM_LAYOUT_REFERENCE) comes from a static device array of QGEMM_STATIC_SCRATCH_BYTES that every GPU the
+ * library runs on holds until the process ends.  The call allocates and frees nothing.  A problem that needs
+ * more returns QGEMM_ERR_SCRATCH_TOO_SMALL and launches nothing.  All calls on one GPU share the array: two
+ * calls whose kernels overlap in time on one GPU (different streams, or threads) race. */
+#define QGEMM_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int qgemm_scaled_gemm_static(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
+                             const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N,
+                             size_t K, int split_k, void *stream);
 
 /* Library workspace (no reference counterpart: the reference's entries take none).  Calls that split K, that
  * take operands or scales in an arrangement the kernels do not read directly, and the per-matrix quantiser keep

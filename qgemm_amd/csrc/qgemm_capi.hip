@@ -23,6 +23,14 @@ using namespace qgemm;
 
 namespace {
 
+// Scratch of the entry point that allocates nothing (qgemm_scaled_gemm_static): split-K partial planes,
+// transposed block scales and transposed operands of one call.  One copy per device, held until the process
+// ends; host code never uses the array's name as an address, only what hipGetSymbolAddress returned for the
+// device that is current (static_scratch_locked).
+constexpr size_t kStaticScratchBytes = QGEMM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+
 struct WsBlock {
     void *p = nullptr;
     size_t bytes = 0;
@@ -44,6 +52,8 @@ struct Context {
     hipStream_t ws_last_stream = nullptr;
     bool ws_event_recorded = false;
     bool ws_used_by_call = false;              // the running entry asked for the workspace
+    bool static_call = false;                  // the running entry takes its workspace from the static scratch
+    void *static_ptr[kMaxDevices] = {};        // device address of `scratch`, per device
     long force_config = -1;     // index into the variant table, -1 = heuristic
     long force_split = 0;       // 0 = heuristic
     long force_group_m = 0;     // 0 = default
@@ -60,6 +70,8 @@ Context g_ctx;
         if (e_ != hipSuccess) return QGEMM_ERR_LAUNCH; \
     } while (0)
 
+int static_scratch_locked(void **out);
+
 int ensure_init_locked() {
     if (g_ctx.ready) return QGEMM_OK;
     int n = 0;
@@ -68,12 +80,29 @@ int ensure_init_locked() {
     HIP_TRY(hipGetDevice(&dev));
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    void *scratch_dev = nullptr;               // address of the static scratch on this device, kept for later
+    int sst = static_scratch_locked(&scratch_dev);
+    if (sst != QGEMM_OK) return sst;
     g_ctx.device = dev;
     g_ctx.num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     // tuning knobs, also reachable through qgemm_set_option
     if (const char *e = std::getenv("QGEMM_FORCE_CONFIG")) g_ctx.force_config = std::atol(e);
     if (const char *e = std::getenv("QGEMM_GROUP_M")) g_ctx.force_group_m = std::atol(e);
     g_ctx.ready = true;
+    return QGEMM_OK;
+}
+
+// Device address of the static scratch on the current device (looked up once per device).
+int static_scratch_locked(void **out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return QGEMM_ERR_UNSUPPORTED;
+    if (!g_ctx.static_ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return QGEMM_ERR_LAUNCH;
+        g_ctx.static_ptr[dev] = p;
+    }
+    *out = g_ctx.static_ptr[dev];
     return QGEMM_OK;
 }
 
@@ -87,12 +116,17 @@ bool stream_is_capturing(hipStream_t stream) {
 }
 
 // Workspace of `bytes` for a call enqueued on `stream`.
-// The library's block, grown when too small.  Growing allocates a new block and retires the old
+//   * qgemm_scaled_gemm_static: the static scratch; larger requests are an error, nothing is allocated.
+//   * otherwise the library's block, grown when too small.  Growing allocates a new block and retires the old
 //     one without freeing it (see Context).  While the stream is being captured into a graph nothing is
 //     allocated and no event is waited for or recorded: a call that would have to grow the block fails with
 //     QGEMM_ERR_ALLOC (the caller reserves the room before the capture, qgemm_reserve_workspace, or runs the
 //     call once eagerly), and ordering replays against other users of the workspace is the caller's business.
 int ensure_workspace_locked(size_t bytes, hipStream_t stream, void **out) {
+    if (g_ctx.static_call) {
+        if (bytes > kStaticScratchBytes) return QGEMM_ERR_SCRATCH_TOO_SMALL;
+        return static_scratch_locked(out);
+    }
     const bool capturing = stream_is_capturing(stream);
     if (bytes > g_ctx.ws.bytes) {
         if (capturing) return QGEMM_ERR_ALLOC;
@@ -674,6 +708,7 @@ QGEMM_EXPORT const char *qgemm_status_string(int status) {
         case QGEMM_ERR_NOT_DIVISIBLE_N: return "N is not divisible by any predefined BLOCK_TILE_SIZE_N in the list";
         case QGEMM_ERR_NOT_DIVISIBLE_K: return "K is not divisible by any predefined BLOCK_TILE_SIZE_K in the list";
         case QGEMM_ERR_TOO_LARGE: return "dimension or stride too large";
+        case QGEMM_ERR_SCRATCH_TOO_SMALL: return "problem needs more than the static scratch (QGEMM_STATIC_SCRATCH_BYTES)";
     }
     return "unknown status";
 }
@@ -895,7 +930,8 @@ QGEMM_EXPORT int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const voi
 
 namespace {
 
-int scaled_gemm_entry(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
+// Body of qgemm_scaled_gemm and qgemm_scaled_gemm_static; `use_static`: the workspace is the static scratch.
+int scaled_gemm_entry(bool use_static, int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
                       const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N, size_t K,
                       int split_k, void *stream_) {
     if (in_dtype != QGEMM_DT_I8 && in_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
@@ -918,6 +954,10 @@ int scaled_gemm_entry(int in_dtype, int out_dtype, int scale_mode, int layout, c
     std::lock_guard<std::mutex> lock(g_ctx.mu);
     int st = ensure_init_locked();
     if (st != QGEMM_OK) return st;
+    struct StaticScope {        // every workspace request of this call goes to the static scratch
+        explicit StaticScope(bool on) { g_ctx.static_call = on; }
+        ~StaticScope() { g_ctx.static_call = false; }
+    } scope(use_static);
     WorkspaceUse ws_use(stream);
 
     const bool block = scale_mode == QGEMM_SCALE_BLOCK128;
@@ -1026,7 +1066,14 @@ extern "C" {
 QGEMM_EXPORT int qgemm_scaled_gemm(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A, const void *B,
                       const float *a_scale, const float *b_scale, void *C, size_t ldC, size_t M, size_t N, size_t K,
                       int split_k, void *stream) {
-    return scaled_gemm_entry(in_dtype, out_dtype, scale_mode, layout, A, B, a_scale, b_scale, C, ldC, M, N, K, split_k,
+    return scaled_gemm_entry(false, in_dtype, out_dtype, scale_mode, layout, A, B, a_scale, b_scale, C, ldC, M, N, K, split_k,
+                             stream);
+}
+
+QGEMM_EXPORT int qgemm_scaled_gemm_static(int in_dtype, int out_dtype, int scale_mode, int layout, const void *A,
+                                          const void *B, const float *a_scale, const float *b_scale, void *C, size_t ldC,
+                                          size_t M, size_t N, size_t K, int split_k, void *stream) {
+    return scaled_gemm_entry(true, in_dtype, out_dtype, scale_mode, layout, A, B, a_scale, b_scale, C, ldC, M, N, K, split_k,
                              stream);
 }
 

@@ -11,7 +11,7 @@ STATUS_OK = 0
 STATUS_NAMES = {
     0: "QGEMM_OK", 1: "QGEMM_ERR_INVALID_ARG", 2: "QGEMM_ERR_UNSUPPORTED", 3: "QGEMM_ERR_NO_DEVICE",
     4: "QGEMM_ERR_LAUNCH", 5: "QGEMM_ERR_ALLOC", 6: "QGEMM_ERR_NOT_DIVISIBLE_M", 7: "QGEMM_ERR_NOT_DIVISIBLE_N",
-    8: "QGEMM_ERR_NOT_DIVISIBLE_K", 9: "QGEMM_ERR_TOO_LARGE",
+    8: "QGEMM_ERR_NOT_DIVISIBLE_K", 9: "QGEMM_ERR_TOO_LARGE", 10: "QGEMM_ERR_SCRATCH_TOO_SMALL",
 }
 
 
@@ -37,6 +37,7 @@ SIGNATURES = {
     "qgemm_status_string": (C.c_char_p, [_i]),
     "qgemm_gemm": (_i, [_i, _i, _i, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp]),
     "qgemm_scaled_gemm": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _i, _vp]),
+    "qgemm_scaled_gemm_static": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _i, _vp]),
     "qgemm_reserve_workspace": (_i, [_sz]),
     "qgemm_workspace_info": (_i, [C.POINTER(_vp), C.POINTER(_sz)]),
     "qgemm_transpose": (_i, [_i, _vp, _vp, _sz, _sz, _vp]),

@@ -169,6 +169,7 @@ def test_too_large_is_reported_not_wrapped():
     assert lib.qgemm_transpose(1, one, one, 4, 1 << 31, None) == 9
     # block scales: M * ceil(K / 128) * 4 bytes >= 2^32 cannot go to the MFMA kernel
     assert Q.plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 1 << 20, 256, 1 << 17) == "strided_any_shape"
+    assert b"static scratch" in lib.qgemm_status_string(10)
 
 
 def test_workspace_entries_need_no_device_to_answer():
