@@ -58,6 +58,47 @@ def _time_launches(fn, steps, warmup):
     return wall, e0.elapsed_time(e1) / steps
 
 
+def _time_each_launch(fn, steps, warmup):
+    """-> (wall ms per step, event ms per launch, [ms of every timed launch]): one HIP event between consecutive
+    launches, so the launch-to-launch period of each timed launch is on record."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(steps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, ev[0].elapsed_time(ev[steps]) / steps, [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
+
+
+def _graph_time(fns, reps=20):
+    """Microseconds per launch of the launches `fns`, captured once into a HIP graph and replayed `reps` times: what
+    a caller that captures its GEMMs sees, without one Python call per 5-microsecond kernel."""
+    import torch
+    for f in fns:
+        f()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for f in fns:
+            f()
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * len(fns))
+
+
 def _quant_fp8(x):
     import torch
     s = (x.abs().max() / 448.0).float().reshape(1)
@@ -148,6 +189,7 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the headline workload")
     ap.add_argument("--cpu-rows", type=int, default=8192, help="rows of C the CPU baseline computes (0 = skip)")
     ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs")
+    ap.add_argument("--no-steady", action="store_true", help="skip the 100 + 200 launch steady-state block")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three plain device copies of 256 MiB (the known-size kernel the FETCH_SIZE / "
                          "WRITE_SIZE counters are scaled against) and exit")
@@ -185,7 +227,7 @@ def main():
     b_q, sb = _quant_fp8(torch.randn(N, K, device=dev))
     c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     run = lambda: Q.scaled_gemm(a_q, b_q, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)
-    wall_ms, ev_ms = _time_launches(run, args.steps, args.warmup)
+    wall_ms, ev_ms, per_launch_ms = _time_each_launch(run, args.steps, args.warmup)
     cfg_name = Q.last_config()
     flops = 2.0 * M * N * K
     tflops_wall = flops / (wall_ms * 1e-3) / 1e12
@@ -203,92 +245,106 @@ def main():
                      "traffic_unit": "bytes per launch (L2 <-> fabric, rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
                      "algorithmic_bytes": float(M * K + N * K + 2 * M * N),
                      "kernel_ms": ev_ms, "flops_per_launch": flops},
+        # launch-to-launch period of every timed launch, in order (HIP events between the launches): on a part that
+        # was idle the first launches run at boost clock, the next ten to twenty well below the clock it settles at
+        "per_launch_ms": [round(t, 4) for t in per_launch_ms],
     }
+    # the same operands, same process, once the power management has settled: 100 untimed + 200 timed launches
+    if not args.no_steady:
+        _, ss_ms = _time_launches(run, 200, 100)
+        out["steady_state"] = {"launches": 200, "warmup": 100, "kernel_ms": ss_ms, "tflops": flops / ss_ms / 1e9,
+                               "frac": flops / ss_ms / 1e9 / PEAK_TFLOPS["f8"]}
 
-    # ---- the other configs (short; parity for them is in tests/)
+    # ---- the other configs (parity for them is in tests/).  One policy for every entry: 10 untimed + 30 timed
+    # launches between two HIP events, after the steady-state block above, i.e. on a part that is warm; shapes
+    # whose kernel is shorter than a Python call (configs 1 and 5) by replaying a captured graph of 24 launches.
     if not args.no_extra:
-        extra = {}
+        XW, XS = 10, 30
+        extra = {"timing": "every entry: %d untimed + %d timed launches between two HIP events, run after the steady-state "
+                           "block; cfg1 and cfg5: microseconds per launch of a captured graph of 24 launches, replayed 20 "
+                           "times" % (XW, XS)}
+        tx = lambda fn: _time_launches(fn, XS, XW)[1]
+
+        def gemm_entry(ms, fl, peak):
+            return {"tflops": fl / ms / 1e9, "frac_of_peak": fl / ms / 1e9 / peak, "ms": ms, "kernel": Q.last_config()}
         ai, sai = _quant_i8(torch.randn(M, K, device=dev))
         bi, sbi = _quant_i8(torch.randn(N, K, device=dev))
         cf = torch.empty(M, N, dtype=torch.float32, device=dev)
-        _, ms = _time_launches(lambda: Q.int8_mm(ai, bi, sai, sbi, cf), max(5, args.steps // 2), 3)
-        extra["int8_per_matrix_%d" % M] = {"tflops": flops / ms / 1e9, "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["i8"],
-                                           "ms": ms, "kernel": Q.last_config()}
+        extra["int8_per_matrix_%d" % M] = gemm_entry(tx(lambda: Q.int8_mm(ai, bi, sai, sbi, cf)), flops, PEAK_TFLOPS["i8"])
         # the same product with bf16 output (half the bytes of C; what the headline's fp8 run writes)
         cb16 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-        _, ms = _time_launches(lambda: Q.int8_mm(ai, bi, sai, sbi, cb16), max(5, args.steps // 2), 3)
-        extra["int8_per_matrix_%d_bf16_out" % M] = {"tflops": flops / ms / 1e9,
-                                                    "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["i8"], "ms": ms,
-                                                    "kernel": Q.last_config()}
+        extra["int8_per_matrix_%d_bf16_out" % M] = gemm_entry(tx(lambda: Q.int8_mm(ai, bi, sai, sbi, cb16)), flops,
+                                                             PEAK_TFLOPS["i8"])
         del ai, bi, cf, cb16
         # cfg 2: int8 4096^3 -> f32
         m2 = 4096
         ai, sai = _quant_i8(torch.randn(m2, m2, device=dev))
         bi, sbi = _quant_i8(torch.randn(m2, m2, device=dev))
         cf = torch.empty(m2, m2, dtype=torch.float32, device=dev)
-        _, ms = _time_launches(lambda: Q.int8_mm(ai, bi, sai, sbi, cf), 20, 3)
-        extra["cfg2_int8_4096"] = {"tflops": 2.0 * m2 ** 3 / ms / 1e9, "ms": ms, "kernel": Q.last_config()}
-        # cfg 1: fp16 1024^3, B stored N x K
+        extra["cfg2_int8_4096"] = gemm_entry(tx(lambda: Q.int8_mm(ai, bi, sai, sbi, cf)), 2.0 * m2 ** 3, PEAK_TFLOPS["i8"])
+        del ai, bi, cf
+        # cfg 1: fp16 1024^3, B stored N x K (launch-bound: graph replay)
         m1 = 1024
         ah = (torch.rand(m1, m1, device=dev) * 2 - 1).half()
         bh = (torch.rand(m1, m1, device=dev) * 2 - 1).half()
         ch = torch.empty(m1, m1, dtype=torch.float16, device=dev)
-        _, ms = _time_launches(lambda: Q.gemm(ah, bh, ch, "nk"), 50, 5)
-        extra["cfg1_fp16_1024"] = {"tflops": 2.0 * m1 ** 3 / ms / 1e9, "ms": ms, "kernel": Q.last_config()}
+        us = _graph_time([lambda: Q.gemm(ah, bh, ch, "nk")] * 24)
+        extra["cfg1_fp16_1024"] = dict(gemm_entry(us * 1e-3, 2.0 * m1 ** 3, PEAK_TFLOPS["f16"]), us_per_launch=us)
         # cfg 4: fp8 block-scaled 6144 x 4608 x 7168
         m4, n4, k4 = 6144, 4608, 7168
+        f4 = 2.0 * m4 * n4 * k4
         a4, _ = _quant_fp8(torch.randn(m4, k4, device=dev))
         b4, _ = _quant_fp8(torch.randn(n4, k4, device=dev))
         as4 = torch.rand(m4, k4 // 128, device=dev) * 1.5 + 0.5
         bs4 = torch.rand(n4 // 128, k4 // 128, device=dev) * 1.5 + 0.5
         c4 = torch.empty(m4, n4, dtype=torch.bfloat16, device=dev)
-        _, ms = _time_launches(lambda: Q.scaled_gemm(a4, b4, as4, bs4, c4, m4, n4, k4, Q.SCALE_BLOCK128), 20, 3)
-        extra["cfg4_fp8_block_6144x4608x7168"] = {"tflops": 2.0 * m4 * n4 * k4 / ms / 1e9, "ms": ms,
-                                                  "frac_of_peak": 2.0 * m4 * n4 * k4 / ms / 1e9 / PEAK_TFLOPS["f8"],
-                                                  "kernel": Q.last_config()}
+        extra["cfg4_fp8_block_6144x4608x7168"] = gemm_entry(
+            tx(lambda: Q.scaled_gemm(a4, b4, as4, bs4, c4, m4, n4, k4, Q.SCALE_BLOCK128)), f4, PEAK_TFLOPS["f8"])
         del a4, b4, c4
-        # cfg 5: skinny split-K, N=7168, K=2048 (bandwidth-bound: report GB/s of algorithmic bytes)
+        # cfg 5: skinny M, N = 7168, K = 2048, int8 (f32 out) and fp8 (bf16 out); bandwidth-bound: GB/s of algorithmic
+        # bytes.  "rotated": every launch of the graph reads another B (24 buffers, 352 MB: more than the Infinity
+        # Cache holds); "resident": all 24 launches read the same B.
         n5, k5 = 7168, 2048
-        for m5 in (16, 64, 128):
-            a5, s5a = _quant_fp8(torch.randn(m5, k5, device=dev))
-            # rotate over enough B buffers to exceed the 256 MB Infinity Cache
-            nbuf = 24
-            b5s = [_quant_fp8(torch.randn(n5, k5, device=dev)) for _ in range(nbuf)]
-            c5 = torch.empty(m5, n5, dtype=torch.bfloat16, device=dev)
-            it = [0]
-
-            def run5():
-                bq, sbq = b5s[it[0] % nbuf]
-                it[0] += 1
-                Q.scaled_gemm(a5, bq, s5a, sbq, c5, m5, n5, k5, Q.SCALE_PER_MATRIX)
-            _, ms = _time_launches(run5, 96, 24)
-            nbytes = n5 * k5 + m5 * k5 + m5 * n5 * 2
-            extra["cfg5_fp8_skinny_M%d" % m5] = {
-                "tflops": 2.0 * m5 * n5 * k5 / ms / 1e9, "GBps": nbytes / ms / 1e6,
-                "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS, "ms": ms, "kernel": Q.last_config()}
+        nbuf = 24
+        for fam in ("fp8", "int8"):
+            quant, out_dt, in_dt = ((_quant_fp8, torch.bfloat16, Q.DT_F8E4M3) if fam == "fp8"
+                                    else (_quant_i8, torch.float32, Q.DT_I8))
+            b5s = [quant(torch.randn(n5, k5, device=dev)) for _ in range(nbuf)]
+            for m5 in (16, 64, 128):
+                a5, s5a = quant(torch.randn(m5, k5, device=dev))
+                c5 = torch.empty(m5, n5, dtype=out_dt, device=dev)
+                mk = lambda bq, sbq: (lambda: Q.scaled_gemm(a5, bq, s5a, sbq, c5, m5, n5, k5, Q.SCALE_PER_MATRIX,
+                                                            in_dtype=in_dt))
+                us_rot = _graph_time([mk(bq, sbq) for (bq, sbq) in b5s])
+                us_res = _graph_time([mk(*b5s[0])] * nbuf)
+                nbytes = n5 * k5 + m5 * k5 + m5 * n5 * c5.element_size()
+                extra["cfg5_%s_skinny_M%d" % (fam, m5)] = {
+                    "us_per_launch_rotated": us_rot, "us_per_launch_resident": us_res,
+                    "GBps": nbytes / us_rot / 1e3, "frac_of_hbm_peak": nbytes / us_rot / 1e3 / PEAK_HBM_GBS,
+                    "GBps_resident": nbytes / us_res / 1e3, "tflops": 2.0 * m5 * n5 * k5 / us_rot / 1e6,
+                    "algorithmic_bytes": nbytes, "kernel": Q.last_config()}
             del b5s
-        # cfg 4 in the reference's own storage (A is K x M, B is K x N, scales [K/128, M] and [K/128, N/128]): read
-        # as it lies through K-major tiles and transposing LDS reads
+        # cfg 4 in the reference's own storage (A is K x M, B is K x N, scales [K/128, M] and [K/128, N/128])
         a4r, _ = _quant_fp8(torch.randn(k4, m4, device=dev))
         b4r, _ = _quant_fp8(torch.randn(k4, n4, device=dev))
         as4r = torch.rand(k4 // 128, m4, device=dev) * 1.5 + 0.5
         bs4r = torch.rand(k4 // 128, n4 // 128, device=dev) * 1.5 + 0.5
         c4r = torch.empty(m4, n4, dtype=torch.bfloat16, device=dev)
-        _, ms = _time_launches(lambda: Q.fp8_mm(a4r.t(), b4r.t(), as4r.t(), bs4r.t(), c4r), 20, 3)
-        extra["cfg4_reference_layout_fp8_mm"] = {"tflops": 2.0 * m4 * n4 * k4 / ms / 1e9, "ms": ms, "kernel": Q.last_config()}
+        extra["cfg4_reference_layout_fp8_mm"] = gemm_entry(
+            tx(lambda: Q.fp8_mm(a4r.t(), b4r.t(), as4r.t(), bs4r.t(), c4r)), f4, PEAK_TFLOPS["f8"])
         del a4r, b4r, c4r
         # transpose utility (HBM-bound: 2 * M * N * element bytes)
         for (mt, nt, dtt, nm) in ((8192, 8192, torch.bfloat16, "2B"), (7168, 6144, torch.uint8, "1B")):
             xt = torch.randint(0, 100, (mt, nt), device=dev).to(dtt)
             yt = torch.empty(nt, mt, dtype=dtt, device=dev)
-            _, ms = _time_launches(lambda: Q.matrix_transpose(xt, yt), 20, 3)
+            ms = tx(lambda: Q.matrix_transpose(xt, yt))
             gbs = 2.0 * mt * nt * xt.element_size() / ms / 1e6
             extra["transpose_%s_%dx%d" % (nm, mt, nt)] = {"GBps": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS, "ms": ms}
         # quantisers (HBM-bound): bytes = input (twice for the two-pass per-matrix form) + one output byte
         xq = torch.randn(m4, k4, device=dev)
         for (mode, nm, passes) in ((Q.QUANT_PER_MATRIX, "per_matrix", 2), (Q.QUANT_BLOCK_1x128, "1x128", 1),
                                    (Q.QUANT_BLOCK_128x128, "128x128", 1)):
-            _, ms = _time_launches(lambda: Q.quantize(xq, torch.float8_e4m3fn, mode), 20, 3)
+            ms = tx(lambda: Q.quantize(xq, torch.float8_e4m3fn, mode))
             gbs = m4 * k4 * (4.0 * passes + 1.0) / ms / 1e6
             extra["quantize_fp8_%s_f32_%dx%d" % (nm, m4, k4)] = {"GBps": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS, "ms": ms}
         del xq
@@ -299,14 +355,10 @@ def main():
         xb = torch.randn(M, K, device=dev).bfloat16()
         yb = torch.randn(N, K, device=dev).bfloat16()
         cb = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-        _, ms = _time_launches(lambda: Q.bf16_mm(xb, yb, cb), 20, 3)
-        extra["bf16_%d" % M] = {"tflops": flops / ms / 1e9, "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["bf16"],
-                                "ms": ms, "kernel": Q.last_config()}
-        # the same product with B stored K x N (the storage of GEMM_kernel_v1..v5): the kernel reads it as it lies
+        extra["bf16_%d" % M] = gemm_entry(tx(lambda: Q.bf16_mm(xb, yb, cb)), flops, PEAK_TFLOPS["bf16"])
+        # the same product with B stored K x N (the storage of GEMM_kernel_v1..v5)
         ybt = yb.t().contiguous()
-        _, ms = _time_launches(lambda: Q.gemm(xb, ybt, cb, "kn"), 20, 3)
-        extra["bf16_nn_%d" % M] = {"tflops": flops / ms / 1e9, "frac_of_peak": flops / ms / 1e9 / PEAK_TFLOPS["bf16"],
-                                   "ms": ms, "kernel": Q.last_config()}
+        extra["bf16_nn_%d" % M] = gemm_entry(tx(lambda: Q.gemm(xb, ybt, cb, "kn")), flops, PEAK_TFLOPS["bf16"])
         del ybt
         # interleaved blocks of ten launches, this library and the vendor's in turn, so both see the same clocks
         def interleaved(ours, theirs, rounds=10, per_block=10):

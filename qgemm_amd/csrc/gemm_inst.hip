@@ -2,6 +2,7 @@
 // per family with -DINST_ARITH=<Arith> -DINST_BLOCK=<0|1> -DINST_FN=<table fn>,
 // so the families build in parallel.
 #include "variants.h"
+#include "gemm_skinny.cuh"
 
 #include <type_traits>
 
@@ -26,6 +27,26 @@ static hipError_t launch_variant(const GemmArgs &a, uint32_t grid, hipStream_t s
     }
     hipLaunchKernelGGL(gemm_nt_kernel<C>, dim3(grid), dim3(C::THREADS), C::LDS_BYTES, s, a);
     return hipGetLastError();
+}
+
+template <class C>
+static hipError_t launch_skinny(const GemmArgs &a, uint32_t grid, hipStream_t s) {
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_skinny_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(gemm_skinny_kernel<C>, dim3(grid), dim3(C::THREADS), C::LDS_BYTES, s, a);
+    return hipGetLastError();
+}
+// row of the skinny-M kernel (gemm_skinny.cuh): 16 * TM rows x 32 columns, eight waves splitting K between them.
+// Picked by choose_variant in place of the narrow simple-pipeline tiles, never by the table scan (auto_ok = false).
+template <int TM>
+static Variant skinny_row(const char *name) {
+    using C = SkinnyCfg<INST_ARITH, TM>;
+    return Variant{name, C::ARITH, false, C::BM, C::BN, C::THREADS, C::LDS_BYTES, LOAD_VGPR, false, 8, &launch_skinny<C>};
 }
 
 #define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) != PIPE_SIMPLE, INST_KMAJ>
@@ -90,6 +111,18 @@ static const Variant kTable[] = {
 #else
     row_of<true, GemmCfg<INST_ARITH, false, 64, 128, 1, 4, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 6, 2>,
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("64x128_w1x4_k2", true),
+#endif
+    // skinny M (gemm_skinny.cuh): the K split inside the workgroup, no staging, no barrier in the K loop
+#if INST_BLOCK || INST_KMAJ      // (no block-scale or K-major form: aliases, so indices agree across families)
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+#else
+    skinny_row<1>("skinny_16x32_k8"),
+    skinny_row<2>("skinny_32x32_k8"),
+    skinny_row<4>("skinny_64x32_k8"),
+    skinny_row<8>("skinny_128x32_k8"),
 #endif
 };
 

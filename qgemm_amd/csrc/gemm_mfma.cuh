@@ -170,6 +170,22 @@ struct GemmCfg {
     static_assert(KMAJ == 0 || PIPE == PIPE_SIMPLE, "K-major tiles: simple pipeline only");
 };
 
+// Time stamps of a measurement build (-DQGEMM_DEBUG_BUILD=1; the library proper compiles them to nothing): up to N
+// readings of the 100 MHz clock all CUs share, written per wave to GemmArgs::dbg_cycles when the kernel ends.
+#if QGEMM_DEBUG_BUILD
+#define QGEMM_STAMP_DECL(N) unsigned long long qgemm_stamp_[N] = {}
+#define QGEMM_STAMP(I) (qgemm_stamp_[I] = __builtin_amdgcn_s_memrealtime())
+#define QGEMM_STAMP_WRITE(PTR, SLOT, N, COND)                                              \
+    do {                                                                                   \
+        if ((PTR) && (COND))                                                               \
+            for (int i_ = 0; i_ < (N); ++i_) (PTR)[(size_t)(SLOT) * (N) + i_] = qgemm_stamp_[i_]; \
+    } while (0)
+#else
+#define QGEMM_STAMP_DECL(N) ((void)0)
+#define QGEMM_STAMP(I) ((void)0)
+#define QGEMM_STAMP_WRITE(PTR, SLOT, N, COND) ((void)0)
+#endif
+
 typedef __attribute__((address_space(3))) void lds_void;
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v2i lds_v2i;

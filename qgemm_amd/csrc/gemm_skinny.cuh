@@ -1,0 +1,282 @@
+// Skinny-M GEMM for gfx950: M <= 128 rows against a long, narrow strip of B, the K split done inside the
+// workgroup.  The "split-K variant for skinny M" of the reference's plan (README.md:28; the unused split_k of
+// src/gemm/sm89_gemm_kernel_v5.cu:319), built for a part where such a shape is bound by how many bytes are in
+// flight, not by arithmetic: B is read exactly once, straight from HBM.
+//
+// A workgroup owns 16*TM rows x 32 columns of C over the whole of K (or over its K slice when the host splits K
+// on top).  Its eight waves take the 128-byte K steps round robin, two steps per wave and round: in round r wave w
+// computes steps 16 r + w and 16 r + 8 + w of the whole tile.  Nothing is shared on the way, so the K loop has no
+// barrier and no wait on another wave.
+//   * Both operands travel global -> LDS with buffer_load ... lds, eight lanes per 128-byte row, rows rotated as
+//     in gemm_nt_kernel (lds_slot), into a ring of twenty 1 KiB slots that belongs to the wave alone, and from
+//     there into registers with conflict-free ds_read_b128 in the MFMA's lane layout.  (Loading the fragments
+//     from global memory straight into that layout was built first and is far slower: neighbouring lanes are
+//     neighbouring rows there, the texture addresser merges nothing, and every 16 bytes become a request of
+//     their own: 64 cycles per instruction and CU.)
+//   * The wave waits for its own copies with s_waitcnt vmcnt(n): copies land in issue order, and the program of a
+//     round is fixed, so every n is a compile-time constant.  All of B of the round (the stream from HBM) is
+//     requested when the round starts; A (shared by every workgroup, an L2 hit) fills what is left of the ring,
+//     is drained into registers as it lands and makes room for the rest of A: two steps of a 128-row tile are
+//     40 KiB, twice the ring.  Steps past the end of K are copied like all others (the buffer range check turns
+//     them into zeros).
+// The eight partial sums meet once, in LDS, and are added in wave order (a fixed order: the same bits every
+// run; exact for int32), then scaled, converted and stored like the epilogue of gemm_nt_kernel.
+#pragma once
+#include "gemm_mfma.cuh"
+
+namespace qgemm {
+
+template <int ARITH_, int TM_>
+struct SkinnyCfg {
+    static constexpr int ARITH = ARITH_;
+    static constexpr int TM = TM_, TN = 2;                  // 16 x 16 MFMA tiles of the workgroup's tile
+    static constexpr int BM = 16 * TM_, BN = 32;
+    static constexpr int NW = 8, THREADS = NW * kWave;
+    static constexpr int SLOTS = 20;                        // ring slots (1 KiB = one copy instruction) per wave
+    static constexpr int SA = 2 * TM, SB = 2 * TN;          // slots of one step of A / of B
+    static constexpr int RING_BYTES = SLOTS * 1024;
+    static constexpr int LDS_BYTES = NW * RING_BYTES;       // the rings; afterwards one partial sum (1 KiB per tile) per wave
+    static_assert(TM == 1 || TM == 2 || TM == 4 || TM == 8, "the programs below are written for these tile heights");
+    static_assert(TM * TN * 1024 <= RING_BYTES, "a wave's partial sums fit its ring");
+};
+
+// all copies of this wave but the last IN_FLIGHT have landed
+template <int IN_FLIGHT>
+__device__ inline void wait_landed() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(IN_FLIGHT));
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <class C>
+__global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    typedef typename AccT<C::ARITH>::type acc_t;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    QGEMM_STAMP_DECL(6);
+    QGEMM_STAMP(0);
+
+    uint32_t wg = blockIdx.x, z = 0;
+    if (p.nsplit > 1) {
+        z = __builtin_amdgcn_readfirstlane(wg % p.nsplit);
+        wg = __builtin_amdgcn_readfirstlane(wg / p.nsplit);
+    }
+    // column strips side by side (the few row tiles of one strip are neighbours: they share the strip of B in L2)
+    const uint32_t tm = __builtin_amdgcn_readfirstlane(wg % p.tiles_m), tn = __builtin_amdgcn_readfirstlane(wg / p.tiles_m);
+    const uint32_t row0 = tm * C::BM, col0 = tn * C::BN;
+    const uint32_t kbeg = z * p.ksteps_per_split;
+    const uint32_t kend = kbeg + p.ksteps_per_split < p.ksteps ? kbeg + p.ksteps_per_split : p.ksteps;
+    const int nk = (int)(kend - kbeg);
+
+    // Buffer resources end with the last valid row of the tile and the last byte of the K slice: rows past M / N and
+    // steps past the end of K read as zeros.
+    const uint32_t a_rows = p.M - row0 < (uint32_t)C::BM ? p.M - row0 : C::BM;
+    const uint32_t b_rows = p.N - col0 < (uint32_t)C::BN ? p.N - col0 : C::BN;
+    const uint32_t kbytes = (uint32_t)nk * 128;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A + (size_t)row0 * p.lda + (size_t)kbeg * 128, (a_rows - 1) * p.lda + kbytes);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B + (size_t)col0 * p.ldb + (size_t)kbeg * 128, (b_rows - 1) * p.ldb + kbytes);
+    // a copy moves 8 rows x 128 bytes; lane l fetches the chunk of row l >> 3 that belongs in 16-byte slot l of
+    // the kilobyte (rotation by the row: see lds_slot)
+    const uint32_t rot = (((lane & 7) - (lane >> 3)) & 7) * 16;
+    const uint32_t voff_a = (lane >> 3) * p.lda + rot, voff_b = (lane >> 3) * p.ldb + rot;
+    char *ring = smem + wave * C::RING_BYTES;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int off0 = lds_slot(fr, fg) * 16, off1 = lds_slot(fr, 4 + fg) * 16;
+
+    // copies: n kilobytes of step kt (rows 8 * first ..) of A or B into ring slots slot, slot + 1, ...
+    auto copy_a = [&](int kt, int first, int n, int slot) {
+#pragma unroll
+        for (int i = 0; i < n; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void *)(ring + (slot + i) * 1024), 16, voff_a,
+                                                     (first + i) * 8 * p.lda + (uint32_t)kt * 128, 0, 0);
+    };
+    auto copy_b = [&](int kt, int slot) {
+#pragma unroll
+        for (int i = 0; i < C::SB; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void *)(ring + (slot + i) * 1024), 16, voff_b,
+                                                     i * 8 * p.ldb + (uint32_t)kt * 128, 0, 0);
+    };
+    // fragments of the two steps of a round: [step][block][half]
+    v4i fa[2][C::TM][2], fb[2][C::TN][2];
+    auto drain_a = [&](int s, int blk0, int nblk, int slot) {       // blocks blk0 .. of step s sit in ring slots slot ..
+#pragma unroll
+        for (int i = 0; i < nblk; ++i) {
+            fa[s][blk0 + i][0] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off0);
+            fa[s][blk0 + i][1] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off1);
+        }
+    };
+    auto drain_b = [&](int s, int slot) {
+#pragma unroll
+        for (int i = 0; i < C::TN; ++i) {
+            fb[s][i][0] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off0);
+            fb[s][i][1] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off1);
+        }
+    };
+    auto drained = [&]() {                                  // the fragment reads are done: their slots may be refilled
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    acc_t acc[C::TM][C::TN];
+#pragma unroll
+    for (int a = 0; a < C::TM; ++a)
+#pragma unroll
+        for (int b = 0; b < C::TN; ++b) acc[a][b] = acc_t{0, 0, 0, 0};
+    auto compute = [&](int s) {
+#pragma unroll
+        for (int b = 0; b < C::TN; ++b)
+#pragma unroll
+            for (int a = 0; a < C::TM; ++a)
+                acc[a][b] = mma128<C::ARITH>(fb[s][b][0], fb[s][b][1], fa[s][a][0], fa[s][a][1], acc[a][b]);
+    };
+
+    // ---- one round = steps k and k + 8 of this wave.  Ring programs by tile height (slots per step: A 2 TM, B 4):
+    //   TM <= 2  (at most 16 slots): everything at once.                 B0 B1 A0 A1
+    //   TM == 4  (24 slots):  A0 B0 B1 A1[0..4)  | A0 drained ->  A1[4..8)
+    //   TM == 8  (40 slots):  A0[0..12) B0 B1    | A0[0..12) drained -> A0[12..16) A1[0..8) | B0 B1 A0[12..16) drained
+    //                         -> A1[8..16)
+    // A goes in front of B where the ring cannot take the round at once: the wait for it then does not include
+    // the trip to HBM, and its slots turn over while B is still on its way.
+    constexpr int SA = C::SA, SB = C::SB;
+    auto start_round = [&](int k) {
+        if constexpr (C::TM <= 2) {
+            copy_b(k, 0);
+            copy_b(k + C::NW, SB);
+            copy_a(k, 0, SA, 2 * SB);
+            copy_a(k + C::NW, 0, SA, 2 * SB + SA);
+        } else if constexpr (C::TM == 4) {
+            copy_a(k, 0, 8, 0);
+            copy_b(k, 8);
+            copy_b(k + C::NW, 12);
+            copy_a(k + C::NW, 0, 4, 16);
+        } else {
+            copy_a(k, 0, 12, 0);
+            copy_b(k, 12);
+            copy_b(k + C::NW, 16);
+        }
+    };
+    // everything of the round into registers, the MFMAs of its first step, and (next: the round after this one
+    // exists) the first copies of the next round as soon as the ring is empty; the MFMAs of the second step last
+    auto finish_round = [&](int k, bool next, bool two) {
+        if constexpr (C::TM <= 2) {
+            wait_landed<SA>();
+            drain_b(0, 0);
+            drain_b(1, SB);
+            drain_a(0, 0, C::TM, 2 * SB);
+            compute(0);
+            wait_landed<0>();
+            drain_a(1, 0, C::TM, 2 * SB + SA);
+        } else if constexpr (C::TM == 4) {
+            wait_landed<12>();
+            drain_a(0, 0, 4, 0);
+            drained();
+            copy_a(k + C::NW, 4, 4, 0);
+            wait_landed<4>();
+            drain_b(0, 8);
+            drain_b(1, 12);
+            drain_a(1, 0, 2, 16);
+            compute(0);
+            wait_landed<0>();
+            drain_a(1, 2, 2, 0);
+        } else {
+            wait_landed<8>();
+            drain_a(0, 0, 6, 0);
+            drained();
+            copy_a(k, 12, 4, 0);
+            copy_a(k + C::NW, 0, 8, 4);
+            wait_landed<8>();
+            drain_b(0, 12);
+            drain_b(1, 16);
+            drain_a(0, 6, 2, 0);
+            drained();
+            copy_a(k + C::NW, 8, 8, 12);
+            compute(0);
+            wait_landed<8>();
+            drain_a(1, 0, 4, 4);
+            wait_landed<0>();
+            drain_a(1, 4, 4, 12);
+        }
+        drained();
+        if (next) start_round(k + 2 * C::NW);
+        if (two) compute(1);
+    };
+    int k = wave;
+    start_round(k);
+    QGEMM_STAMP(1);
+    for (; k < nk; k += 2 * C::NW) finish_round(k, k + 2 * C::NW < nk, k + C::NW < nk);
+    // (a wave without a step has copies of zeros on their way into its ring, which now takes the partial sums)
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0) & 0xF0FF);
+    __builtin_amdgcn_sched_barrier(0);
+    QGEMM_STAMP(3);
+
+    // ---- the eight partial sums meet in LDS: partial of wave w, tile t at smem + w * RING_BYTES + t * 1 KiB, lane-linear
+    constexpr int T = C::TM * C::TN;
+    char *mine = ring + lane * 16;
+#pragma unroll
+    for (int a = 0; a < C::TM; ++a)
+#pragma unroll
+        for (int b = 0; b < C::TN; ++b) *(acc_t *)(mine + (a * C::TN + b) * 1024) = acc[a][b];
+    __syncthreads();
+    QGEMM_STAMP(4);
+
+    float scale = 1.0f;
+    if (p.per_matrix_scale) scale = p.as[0] * p.bs[0];
+    char *Cz = p.C + (size_t)z * p.split_stride * dtype_bytes(p.out_dtype);
+    // wave w finishes tiles w, w + 8, ...
+#pragma unroll
+    for (int i = 0; i < (T + C::NW - 1) / C::NW; ++i) {
+        const int t = wave + i * C::NW;
+        if (t >= T) break;
+        acc_t s = *(const acc_t *)(smem + (size_t)t * 1024 + lane * 16);
+#pragma unroll
+        for (int w = 1; w < C::NW; ++w) {
+            const acc_t o = *(const acc_t *)(smem + (size_t)w * C::RING_BYTES + (size_t)t * 1024 + lane * 16);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[r] += o[r];
+        }
+        const int a = t / C::TN, b = t % C::TN;
+        const uint32_t m = row0 + a * 16 + (lane & 15);
+        const uint32_t n = col0 + b * 16 + (lane >> 4) * 4;
+        if (m >= p.M || n >= p.N) continue;
+        const size_t idx = (size_t)m * p.ldc + n;
+        const bool full = p.vec_store && n + 3 < p.N;
+        if constexpr (C::ARITH == AR_I8) {
+            if (p.out_dtype == QGEMM_DT_I32) {
+                int *dst = (int *)Cz + idx;
+                if (full) *(v4i *)dst = s;
+                else
+                    for (int r = 0; r < 4; ++r)
+                        if (n + r < p.N) dst[r] = s[r];
+                continue;
+            }
+        }
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = (float)s[r] * scale;
+        if (p.out_dtype == QGEMM_DT_F32) {
+            float *dst = (float *)Cz + idx;
+            if (full) *(v4f *)dst = v4f{v[0], v[1], v[2], v[3]};
+            else
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < p.N) dst[r] = v[r];
+        } else {
+            unsigned short h[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                h[r] = p.out_dtype == QGEMM_DT_BF16 ? f32_to_bf16_bits(v[r]) : f32_to_f16_bits(v[r]);
+            unsigned short *dst = (unsigned short *)Cz + idx;
+            if (full) *(us4 *)dst = us4{h[0], h[1], h[2], h[3]};
+            else
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < p.N) dst[r] = h[r];
+        }
+    }
+    QGEMM_STAMP(5);
+    QGEMM_STAMP_WRITE(p.dbg_cycles, blockIdx.x * C::NW + wave, 6, lane == 0);
+#endif
+}
+
+}  // namespace qgemm

@@ -57,6 +57,9 @@ struct Context {
     long force_config = -1;     // index into the variant table, -1 = heuristic
     long force_split = 0;       // 0 = heuristic
     long force_group_m = 0;     // 0 = default
+#if QGEMM_DEBUG_BUILD
+    long dbg_ptr = 0;           // measurement builds: device buffer for the kernels' time stamps (GemmArgs::dbg_cycles)
+#endif
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes
     std::string last_config;
@@ -289,9 +292,33 @@ int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t kst
     return best;
 }
 
+int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
+                bool may_split, uint32_t *nsplit_out);
+
+// The skinny-M kernel (gemm_skinny.cuh: the K split inside the workgroup, eight waves each on every eighth K step)
+// takes over from the narrow simple-pipeline tiles where it is faster: one row tile (M <= 128), a strip of 32
+// columns per workgroup as the tile choice below would have it, and enough K steps for the eight waves (two each;
+// one each is enough up to 16 rows).  Graph replays over rotated B, fp8, microseconds per launch, narrow tile
+// against skinny kernel: 16 x 7168 x 2048 7.6 / 5.4, 64 x 7168 x 2048 9.0 / 6.7, 128 x 7168 x 2048 11.0 / 8.2,
+// 16 x 7168 x 8192 24.6 / 15.2, 32 x 4096 x 4096 12.7 / 8.3, 128 x 4096 x 4096 18.3 / 12.5, 16 x 1024 x 1024
+// 5.6 / 3.1; with K = 1024 and more than 16 rows or K = 512 the narrow tiles stay ahead (64 x 8192 x 1024 5.0 / 5.2,
+// 128 x 7168 x 512 4.6 / 6.0).  It never wants a K split on top: one makes it slower wherever it was tried.
 // kmaj: the table is a K-major family, which has no narrow tiles: the estimate then serves every M
 int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
                    bool may_split, uint32_t *nsplit_out) {
+    const int vi = choose_tile(tab, count, M, N, ksteps, block, kmaj, cus, may_split, nsplit_out);
+    if (vi < 0 || block || kmaj || M > 128 || tab[vi].bn != 32 || tab[vi].kgroups != 1) return vi;
+    if (ksteps < 8 || (ksteps < 16 && M > 16)) return vi;
+    for (int i = 0; i < count; ++i)
+        if (tab[i].kgroups == 8 && (size_t)tab[i].bm >= M) {        // (rows of the table in ascending height)
+            *nsplit_out = 1;
+            return i;
+        }
+    return vi;
+}
+
+int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
+                bool may_split, uint32_t *nsplit_out) {
     *nsplit_out = 0;                                       // 0: no opinion, plan_nt decides
     if (M > 64 || kmaj) {
         int vi = choose_by_cost(tab, count, M, N, ksteps, block, cus, may_split, nsplit_out);
@@ -500,6 +527,9 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
     a.as_ks = q.as_ks;
     a.bs_ns = q.bs_ns;
     a.bs_ks = q.bs_ks;
+#if QGEMM_DEBUG_BUILD
+    a.dbg_cycles = (unsigned long long *)g_ctx.dbg_ptr;
+#endif
     const bool i32_acc = q.arith == AR_I8;
     if (a.nsplit == 1) {
         a.C = (char *)q.C;
@@ -728,6 +758,9 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "force_split")) g_ctx.force_split = value;
     else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
     else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
+#if QGEMM_DEBUG_BUILD
+    else if (!std::strcmp(key, "dbg_ptr")) g_ctx.dbg_ptr = value;
+#endif
     else if (!std::strcmp(key, "row_split")) g_ctx.row_split = value;
     else return QGEMM_ERR_INVALID_ARG;
     return QGEMM_OK;

@@ -13,7 +13,8 @@ struct Variant {
     bool block_scale;
     int bm, bn, threads, lds_bytes, loader;
     bool auto_ok;   // the shape heuristic may pick this row (the others are reachable through force_config)
-    int kgroups;    // 2: two sets of waves per workgroup, each computing every other K step (GemmCfg::KG)
+    int kgroups;    // 2: two sets of waves per workgroup, each computing every other K step (GemmCfg::KG);
+                    // 8: the skinny-M kernel, eight waves each computing every eighth K step (gemm_skinny.cuh)
     hipError_t (*launch)(const GemmArgs &, uint32_t grid, hipStream_t);
 };
 

@@ -25,7 +25,9 @@ class QgemmError(RuntimeError):
 
 
 def library_path():
-    return os.path.join(_HERE, _LIB_NAME)
+    """QGEMM_LIBRARY names another build of the library (e.g. the measurement build `make DEBUG=1` leaves as
+    libqgemm_dbg.so); default: libqgemm.so beside this file."""
+    return os.environ.get("QGEMM_LIBRARY") or os.path.join(_HERE, _LIB_NAME)
 
 
 # every symbol include/qgemm.h declares: name -> (restype, argtypes)

@@ -101,9 +101,17 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_BF16, 0, 0, 8192, 4096, 4096) == "256x256_w2x2_solo"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "256x256_w2x2_solo"  # config 3
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8"  # config 4
-    for m, name in ((16, "16x32_w1x2_dma"), (64, "64x32_w4x1_dma"), (128, "128x32_w4x1_dma")):   # config 5
+    # config 5: the skinny-M kernel (K split over the eight waves of a workgroup)
+    for m, name in ((16, "skinny_16x32_k8"), (64, "skinny_64x32_k8"), (128, "skinny_128x32_k8")):
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
         assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
+    assert plan(Q.DT_BF16, 0, 0, 24, 4096, 4096) == "skinny_32x32_k8"
+    # ... but not with few K steps, with block scales, or where the estimate prefers wide tiles
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 7168, 512) == "128x32_w4x1_dma"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 8192, 1024) == "64x32_w4x1_dma"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 1024, 1024) == "skinny_16x32_k8"
+    assert "skinny" not in plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 64, 7168, 2048)
+    assert "skinny" not in plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 28672, 4096)
     # mid sizes: the cost estimate prefers 128 x 128 tiles while they fit in one round of two per CU, and the
     # form with two K groups per workgroup where there are no more tiles than CUs
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 1536, 1536, 1536) == "128x128_w2x2_k2"
