@@ -46,7 +46,7 @@ static hipError_t launch_skinny(const GemmArgs &a, uint32_t grid, hipStream_t s)
 template <int TM>
 static Variant skinny_row(const char *name) {
     using C = SkinnyCfg<INST_ARITH, TM>;
-    return Variant{name, C::ARITH, false, C::BM, C::BN, C::THREADS, C::LDS_BYTES, LOAD_VGPR, false, 8, &launch_skinny<C>};
+    return Variant{name, C::ARITH, false, C::BM, C::BN, C::THREADS, C::LDS_BYTES, LOAD_DMA, false, 8, false, &launch_skinny<C>};
 }
 
 #define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) != PIPE_SIMPLE, INST_KMAJ>
@@ -63,7 +63,7 @@ template <bool OK, class C, class Fallback>
 static Variant row_of(const char *name, bool auto_ok) {
     using P = std::conditional_t<OK, C, Fallback>;
     return Variant{OK ? name : "128x128_w2x2_dma", P::ARITH, P::BLOCK_SCALE, P::BM, P::BN, P::THREADS, P::LDS_BYTES,
-                   P::LOADER, OK && auto_ok, P::KG, &launch_variant<P>};
+                   P::LOADER, OK && auto_ok, P::KG, P::ASK, &launch_variant<P>};
 }
 #define ROWP(NAME, BM, BN, WM_, WN_, LD, PP, AUTO) \
     row_of<kmajor_can(BM, BN, (WM_) * (WN_), PP), CFG(BM, BN, WM_, WN_, LD, PP), CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>(NAME, AUTO)
@@ -123,6 +123,15 @@ static const Variant kTable[] = {
     skinny_row<2>("skinny_32x32_k8"),
     skinny_row<4>("skinny_64x32_k8"),
     skinny_row<8>("skinny_128x32_k8"),
+#endif
+    // the block-scaled 8-wave solo kernel reading a_scale with the K blocks contiguous, as QGEMM_LAYOUT_K_CONTIGUOUS
+    // passes it (GemmCfg::ASK): launch_nt swaps it in for the row above of the same name when the scales allow it,
+    // which saves the transposed copy of a_scale that the other kernels need
+#if INST_BLOCK && !INST_KMAJ
+    row_of<true, GemmCfg<INST_ARITH, true, 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, 0, true, 0, 0, 1, true>,
+           CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("256x256_w2x4_solo8_ks", false),
+#else
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #endif
 };
 

@@ -97,8 +97,13 @@ enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1, PIPE_SOLO = 2 };
 // the A copy of tile k+2 is started two K steps ahead and only the B half of a tile has to
 // land within one step.
 template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int LOADER_ = LOAD_DMA,
-          int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false, int KMAJ_ = 0, int STAGES_ = 0, int KGROUPS_ = 1>
+          int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false, int KMAJ_ = 0, int STAGES_ = 0, int KGROUPS_ = 1,
+          bool ASK_ = false>
 struct GemmCfg {
+    // ASK (block scales, solo pipeline): a_scale is read with the K blocks contiguous, a_scale[m * as_ms + kb], the
+    // arrangement of QGEMM_LAYOUT_K_CONTIGUOUS, instead of rows contiguous, a_scale[m + kb * as_ks].  A compile-time
+    // choice: as a branch inside the K loop it cost the 8-wave kernel 758 spilled registers.
+    static constexpr bool ASK = ASK_;
     // STAGES (simple pipeline, DMA loader): number of LDS stages, 0 = chosen below.
     // KGROUPS = 2: the workgroup has two sets of WAVES_M x WAVES_N waves; all of them copy, set 0 computes the
     // even K steps and set 1 the odd ones of the same tile (one barrier per pair of steps), and the two partial
@@ -168,6 +173,7 @@ struct GemmCfg {
     // tell that they target another buffer.  The simple pipeline issues the next stage's copies behind the reads
     // of a step, so nothing is in flight there; the pipelined schedules live on copies in flight and would stall.
     static_assert(KMAJ == 0 || PIPE == PIPE_SIMPLE, "K-major tiles: simple pipeline only");
+    static_assert(!ASK_ || (BLOCK_SCALE_ && PIPE_ == PIPE_SOLO), "K-contiguous a_scale: block scales, solo pipeline");
 };
 
 // Time stamps of a measurement build (-DQGEMM_DEBUG_BUILD=1; the library proper compiles them to nothing): up to N
@@ -398,10 +404,11 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const int bp0 = (lane & 15) * 4;
     __amdgpu_buffer_rsrc_t ras = make_rsrc(p.as, 0);
     if constexpr (C::BLOCK_SCALE) {
-        // rows contiguous, p.as_ks floats from one K block to the next (p.as_ks > p.M when the rows are part of a
-        // taller matrix)
-        ras = make_rsrc(p.as, ((p.ksteps - 1) * p.as_ks + p.M) * 4);
-        as_voff = (row0 + wm * C::WM + lane) * 4;
+        // rows contiguous (as_ms == 1), p.as_ks floats from one K block to the next (p.as_ks > p.M when the rows
+        // are part of a taller matrix); or, solo pipeline only, K blocks contiguous (as_ks == 1), as_ms floats from
+        // one row to the next
+        ras = make_rsrc(p.as, ((p.ksteps - 1) * p.as_ks + (p.M - 1) * p.as_ms + 1) * 4);
+        as_voff = (row0 + wm * C::WM + lane) * p.as_ms * 4;
 #pragma unroll
         for (int j = 0; j < NBS; ++j) {
             uint32_t nb = (col0 + wn * C::WN) / 128 + j;
@@ -598,12 +605,48 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // the other; v_permlane32_swap: upper half against lower half).  The same pick through ds_bpermute
             // shares the LDS queue, which answers in order, with the fragment reads issued two rows ahead: waiting
             // for a pick then means waiting for those reads as well (7 % of the K loop on config 4).
+            // a_scale as the caller has it, K blocks contiguous (GemmCfg::ASK; the host picks that kernel only with an
+            // even number of K blocks per row and per K slice and 8-byte aligned rows): lane l fetches the scales of
+            // two K blocks of its row at once, on every other step, so the 64 rows of a load, 64 requests of their
+            // own, cost the texture addresser half of what one strided dword per step would.  Either way block kb
+            // sits in component kb & 1 of as_pair.
             float as_b[TMs], bs_c[NBS], sc[2][NBS];
-            auto rotate_scales = [&]() {
+            v2i as_pair[NLD];
+            constexpr bool as_kcont = C::ASK;
+            auto fetch_a_scales = [&](int kt, int comp) {      // for K step kt (of this slice; comp = kt & 1)
+                if constexpr (C::BLOCK_SCALE && !(DBG & 256)) {
+                    const uint32_t kb = kbeg + kt;
+                    if (as_kcont) {
+                        if (comp == 0) {
+#pragma unroll
+                            for (int j = 0; j < NLD; ++j)
+                                as_pair[j] = __builtin_bit_cast(
+                                    v2i, __builtin_amdgcn_raw_buffer_load_b64(ras, as_voff, (64 * j * p.as_ms + kb) * 4, 0));
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < NLD; ++j)
+                            as_pair[j][comp] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (64 * j + kb * p.as_ks) * 4, 0);
+                    }
+                }
+            };
+            auto fetch_b_scales = [&](int kt) {
+                if constexpr (C::BLOCK_SCALE && !(DBG & 256)) {
+                    // (one step past the end of K is fetched like the others: keep that read inside the array)
+                    const uint32_t kb = kbeg + kt, kbc = kb < p.ksteps ? kb : p.ksteps - 1;
+#pragma unroll
+                    for (int j = 0; j < NBS; ++j) bs_raw[j] = p.bs[bs_off[j] + kbc * p.bs_ks];
+                }
+            };
+            // With one b_scale per wave tile and K block (NBS == 1) the factor a_scale * b_scale is formed here, on
+            // the two registers the loads brought, instead of once per row of MFMAs: the same product, the same bits.
+            auto rotate_scales = [&](int comp) {
                 if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
                     for (int j = 0; j < NLD; ++j) {
-                        const unsigned x = (DBG & 256) ? __builtin_bit_cast(unsigned, 1.0f) : (unsigned)as_raw[j];
+                        unsigned x = (DBG & 256) ? __builtin_bit_cast(unsigned, 1.0f) : (unsigned)as_pair[j][comp];
+                        if constexpr (NBS == 1 && !(DBG & 256))
+                            x = __builtin_bit_cast(unsigned, __builtin_bit_cast(float, x) * bs_raw[0]);
                         const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);      // (R0 R0 R2 R2), (R1 R1 R3 R3)
                         const auto e = __builtin_amdgcn_permlane32_swap(r[0], r[0], false, false);  // all R0, all R2
                         const auto o = __builtin_amdgcn_permlane32_swap(r[1], r[1], false, false);  // all R1, all R3
@@ -643,7 +686,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // every other step: the buffer range check turns what lies beyond the operand into zeros, the
             // rest is data nobody reads, and one straight-line loop body serves all steps (a second, guarded
             // copy of the body cost register spills of its own).
-            auto step = [&](int kt) {
+            auto step = [&](int kt, int par) {             // par = kt & 1
                 const int a_nx = next_buf(a_rd);
                 constexpr bool copies = true;
                 // block scales of this step (fetched one step ahead) and the fetch for the next one, in front of
@@ -654,7 +697,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // MFMA of row a-1, the multiply behind the second MFMA of row a, so two factors are live at a time.
                 constexpr int BEHIND = 2;      // MFMAs between a partial product and its fold
                 v4f part[BEHIND + 1];
-                fetch_scales(kt + 1);
+                fetch_a_scales(kt + 1, par ^ 1);
+                fetch_b_scales(kt + 1);
                 auto fold = [&](int i) {
                     if constexpr (C::BLOCK_SCALE && !(DBG & 1) && !(DBG & 128)) {
                         const int pa = i / C::TN, pb = i % C::TN;
@@ -706,7 +750,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                             side(b);
                             if (b == 1) {        // factor of this row, first used behind the next MFMA
 #pragma unroll
-                                for (int j = 0; j < NBS; ++j) sc[a % 2][j] = as_b[a] * bs_c[j];
+                                for (int j = 0; j < NBS; ++j) sc[a % 2][j] = NBS == 1 ? as_b[a] : as_b[a] * bs_c[j];
                             }
                             __builtin_amdgcn_sched_barrier(0);
                             if (i >= BEHIND) fold(i - BEHIND);
@@ -746,15 +790,16 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
                     for (int i = TMs * C::TN - BEHIND; i < TMs * C::TN; ++i) fold(i);
-                    rotate_scales();
+                    rotate_scales(par ^ 1);
                 }
                 a_rd = a_nx;
                 a_wr = next_buf(a_wr);
             };
             if (nk > 0) {
                 if constexpr (C::BLOCK_SCALE) {
-                    fetch_scales(0);
-                    rotate_scales();
+                    fetch_a_scales(0, 0);
+                    fetch_b_scales(0);
+                    rotate_scales(0);
                 }
 #pragma unroll
                 for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
@@ -786,13 +831,17 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         for (int j = 0; j < 6; ++j) {
                             a_rd = j % 3;
                             a_wr = (j + 2) % 3;
-                            step(kt + j);
+                            step(kt + j, j & 1);
                         }
                     }
                     a_rd = 0;            // kt is a multiple of six here
                     a_wr = 2;
                 }
-                for (; kt < nk; ++kt) step(kt);
+                for (; kt + 2 <= nk; kt += 2) {
+                    step(kt, 0);
+                    step(kt + 1, 1);
+                }
+                if (kt < nk) step(kt, 0);
                 __builtin_amdgcn_s_waitcnt(0x0070);      // copies landed, reads done, before LDS serves the epilogue
                 phase_barrier();
                 // the MFMAs above are opaque to the compiler's hazard handling: give the last one its wait states

@@ -582,6 +582,33 @@ int launch_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t
 // arrangement, hip_mix_gemm_kernel.cpp:149): 64 rows of one K block are one 256-byte request.  Scales
 // given with K contiguous (a_scale[m*KB + kb]) are brought to that form first: M*KB floats, a few
 // microseconds.  `room` is where in the workspace the copy goes.
+// Which arrangement of a_scale the kernels of a block-scaled plan read.  Most want it rows-contiguous
+// (a_scale[m + kb * ld], what QGEMM_LAYOUT_REFERENCE passes); the block-scaled 8-wave solo kernel has a twin
+// (GemmCfg::ASK, table name "<name>_ks") that reads it with the K blocks contiguous, as QGEMM_LAYOUT_K_CONTIGUOUS
+// passes it, two K blocks per load: rows 8-byte aligned, an even number of K blocks per row and per K slice.
+// Puts the right one of each pair into the plan.  Returns true when the plan then reads q's scales as they are,
+// false when they first have to be copied rows-contiguous (scales_rows_contiguous).
+bool settle_scale_layout(const NtProblem &q, Plan &pl) {
+    if (!q.block) return true;
+    int count = 0;
+    const Variant *tab = table_for(q.arith, q.block, q.kmaj, &count);
+    auto partner = [&](const Variant *v, bool ks) -> const Variant * {      // the row of the pair with / without ASK
+        if (v->a_scale_k_contiguous == ks) return v;
+        std::string want = v->name;
+        if (ks) want += "_ks";
+        else if (want.size() > 3) want.resize(want.size() - 3);
+        for (int i = 0; tab && i < count; ++i)
+            if (tab[i].a_scale_k_contiguous == ks && want == tab[i].name) return &tab[i];
+        return nullptr;
+    };
+    bool ks = q.as_ms != 1 && q.as_ks == 1 && q.as_ms % 2 == 0 && ((uintptr_t)q.as & 7u) == 0;
+    for (const Plan *p = &pl; ks && p; p = p->rest.get())
+        ks = partner(p->v, true) && !(p->a.nsplit > 1 && p->a.ksteps_per_split % 2 != 0);
+    for (Plan *p = &pl; p; p = p->rest.get())
+        if (const Variant *v = partner(p->v, ks)) p->v = v;
+    return ks || q.as_ms == 1;
+}
+
 int scales_rows_contiguous(NtProblem &q, void *room, hipStream_t stream) {
     if (!q.block || q.as_ms == 1) return QGEMM_OK;
     const size_t KB = (q.Kbytes + 127) / 128;
@@ -602,7 +629,8 @@ int launch_nt(NtProblem q, hipStream_t stream) {
     int st = plan_nt(q, pl);
     if (st != QGEMM_OK) return st;
     void *ws = nullptr;
-    const size_t split_room = (pl.split_bytes + 255) / 256 * 256, as_room = scales_room(q);
+    const size_t split_room = (pl.split_bytes + 255) / 256 * 256;
+    const size_t as_room = settle_scale_layout(q, pl) ? 0 : scales_room(q);
     if (split_room + as_room) {
         st = ensure_workspace_locked(split_room + as_room, stream, &ws);
         if (st != QGEMM_OK) return st;
@@ -812,6 +840,12 @@ QGEMM_EXPORT int qgemm_plan(int in_dtype, int scale_mode, int k_major, size_t M,
     Plan pl;
     const int st = plan_nt(q, pl);
     if (st != QGEMM_OK) return st;
+    if (q.block) {          // dense scales in the arrangement of the layout asked about
+        const uint32_t KB = (uint32_t)((K + 127) / 128);
+        if (k_major == 3) { q.as_ms = 1; q.as_ks = (uint32_t)M; }
+        else { q.as_ms = KB; q.as_ks = 1; }
+        (void)settle_scale_layout(q, pl);
+    }
     name += std::string(pl.v->name) + kmaj_suffix(q.kmaj);
     if (pl.a.nsplit > 1) name += "_splitk" + std::to_string(pl.a.nsplit);
     if (pl.rest) {
@@ -1064,6 +1098,7 @@ int scaled_gemm_entry(bool use_static, int in_dtype, int out_dtype, int scale_mo
         }
         q.A = at;
         q.B = bt;
+        (void)settle_scale_layout(q, pl);            // (scales are rows-contiguous in this layout)
         return run_nt(q, pl, ws, stream);
     }
 

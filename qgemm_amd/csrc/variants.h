@@ -15,6 +15,8 @@ struct Variant {
     bool auto_ok;   // the shape heuristic may pick this row (the others are reachable through force_config)
     int kgroups;    // 2: two sets of waves per workgroup, each computing every other K step (GemmCfg::KG);
                     // 8: the skinny-M kernel, eight waves each computing every eighth K step (gemm_skinny.cuh)
+    bool a_scale_k_contiguous;   // block scales: the kernel also reads a_scale[m * ld + kb] as the caller has it
+                                 // (the others want it rows-contiguous, a_scale[m + kb * ld])
     hipError_t (*launch)(const GemmArgs &, uint32_t grid, hipStream_t);
 };
 

@@ -100,7 +100,9 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x4_solo8"
     assert plan(Q.DT_BF16, 0, 0, 8192, 4096, 4096) == "256x256_w2x2_solo"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "256x256_w2x2_solo"  # config 3
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8"  # config 4
+    # config 4: the twin of the 8-wave kernel that reads a_scale as this layout passes it (56 K blocks per row: even)
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8_ks"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168 - 128) == "256x256_w2x4_solo8"
     # config 5: the skinny-M kernel (K split over the eight waves of a workgroup)
     for m, name in ((16, "skinny_16x32_k8"), (64, "skinny_64x32_k8"), (128, "skinny_128x32_k8")):
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name

@@ -14,7 +14,7 @@ from tests.util import (assert_close, dev, fp8_inputs, fp8_tensor, host, int8_in
 
 pytestmark = pytest.mark.gpu
 
-N_VARIANTS = 22         # rows of the variant table in qgemm_amd/csrc/gemm_inst.hip
+N_VARIANTS = 23         # rows of the variant table in qgemm_amd/csrc/gemm_inst.hip
 
 
 @pytest.fixture(autouse=True)
@@ -168,6 +168,36 @@ def test_fp8_block_scaled_power_of_two_scales_bit_exact(variant, shape):
     c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K,
                   Q.SCALE_BLOCK128, split_k=1 if variant >= 0 else 0)
+    assert np.array_equal(host(c), ref), Q.last_config()
+
+
+@pytest.mark.parametrize("case", [(512, 512, 1024, 0, True), (300, 520, 768, 0, True), (256, 256, 1536, 2, True),
+                                  (256, 256, 1280, 2, False), (256, 256, 384, 0, False), (512, 256, 7168, 0, True)])
+def test_fp8_block_scaled_k_contiguous_scale_twin(case):
+    """The block-scaled 8-wave kernel reads a_scale as QGEMM_LAYOUT_K_CONTIGUOUS passes it (two K blocks per load)
+    when every row holds an even number of K blocks and every K slice an even number of steps, and falls back to
+    a rows-contiguous copy otherwise; bit-exact either way on small integers and power-of-two scales, so a scale
+    taken from the wrong K block or row cannot pass."""
+    M, N, K, split, twin = case
+    say("fp8 block, K-contiguous a_scale", case)
+    rng = np.random.default_rng(17)
+    a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+    as_ = (2.0 ** rng.integers(-3, 4, size=(M, K // 128))).astype(np.float32)
+    bs = (2.0 ** rng.integers(-3, 4, size=((N + 127) // 128, K // 128))).astype(np.float32)
+    ref = R.gemm_fp8_block(a, b, as_, bs)
+    Q.set_option("force_config", 12)
+    Q.set_option("force_split", split)
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
+    assert ("solo8_ks" in Q.last_config()) == twin, Q.last_config()
+    assert np.array_equal(host(c), ref), Q.last_config()
+    # scales whose rows are not 8-byte aligned: the copy again
+    as_off = torch.zeros(as_.size + 1, dtype=torch.float32, device="cuda")
+    as_off[1:] = dev(as_).flatten()
+    c.zero_()
+    Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), as_off[1:], dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
+    assert "solo8_ks" not in Q.last_config()
     assert np.array_equal(host(c), ref), Q.last_config()
 
 
