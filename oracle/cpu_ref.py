@@ -16,10 +16,13 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libcpu_ref.so")
+# QGEMM_ORACLE_LIB names another build of the same source (the sanitizer build of `make -C oracle asan`)
+_LIB_PATH = os.environ.get("QGEMM_ORACLE_LIB") or os.path.join(_HERE, "libcpu_ref.so")
 
 
 def build(force=False):
+    if os.environ.get("QGEMM_ORACLE_LIB"):
+        return _LIB_PATH
     if force or not os.path.exists(_LIB_PATH):
         subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "libcpu_ref.so"])
     return _LIB_PATH
