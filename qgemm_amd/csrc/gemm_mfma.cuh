@@ -66,7 +66,7 @@ struct GemmArgs {
     int out_dtype;        // qgemm_dtype_t of C
     int per_matrix_scale; // multiply by as[0]*bs[0] in the epilogue
     int vec_store;        // 0: scalar stores; 1: C and ldc allow 4-element vector stores; 2: also 16-byte row pieces
-    unsigned long long *dbg_cycles;   // DBG bit 3 builds only: per workgroup {start, loop start, loop end, end}
+    unsigned long long *dbg_cycles;   // measurement builds only (QGEMM_STAMP): time stamps per wave
 };
 
 // How a stage travels from global memory to LDS.
@@ -272,25 +272,13 @@ __device__ inline void mma128_inplace(v4i x0, v4i x1, v4i y0, v4i y1, typename A
     }
 }
 
-// Time stamp of the DBG & 8 builds: shader cycles (per CU, not comparable between CUs), or with DBG bit 5 the
-// constant 100 MHz counter that all CUs share.
-template <int DBG>
-__device__ inline unsigned long long dbg_stamp() {
-    if constexpr (DBG & 32) return __builtin_amdgcn_s_memrealtime();
-    else return __builtin_readcyclecounter();
-}
-
-// DBG is a measurement aid for kernel bring-up; the library only instantiates DBG = 0.  Bits: 1 skip the
-// MFMAs, 2 skip the global loads, 4 skip the fragment reads, 8 per-workgroup time stamps (32: on the shared
-// 100 MHz clock), 16 per-phase cycle sums (ping-pong), 64 no barrier (solo), 128 no block-scale fold,
-// 256 constant block scales (no fetch).  Results are wrong with any of 1 .. 4, 64 .. 256.
-template <class C, int DBG = 0>
+template <class C>
 __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     typedef typename AccT<C::ARITH>::type acc_t;
-    unsigned long long dbg_t0 = 0, dbg_t1 = 0, dbg_t2 = 0;
-    if constexpr (DBG & 8) dbg_t0 = dbg_stamp<DBG>();
+    QGEMM_STAMP_DECL(4);               // start, K loop start, K loop end, end
+    QGEMM_STAMP(0);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -417,7 +405,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     }
     auto fetch_scales = [&](int kt) {          // start the loads for K step kt
-        if constexpr (C::BLOCK_SCALE && !(DBG & 256)) {
+        if constexpr (C::BLOCK_SCALE) {
             const uint32_t kb = kbeg + kt;
 #pragma unroll
             for (int j = 0; j < NLD; ++j)
@@ -429,12 +417,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     };
     auto expand_scales = [&]() {               // what fetch_scales brought becomes as_cur / bs_cur
-        if constexpr (C::BLOCK_SCALE && (DBG & 256)) {
-#pragma unroll
-            for (int a = 0; a < C::TM; ++a) as_cur[a] = 1.0f;
-#pragma unroll
-            for (int j = 0; j < NBS; ++j) bs_cur[j] = 1.0f;
-        } else if constexpr (C::BLOCK_SCALE) {
+        if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
             for (int a = 0; a < C::TM; ++a)
                 as_cur[a] = __builtin_bit_cast(
@@ -489,7 +472,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     };
 
     // ---- K loop
-    if constexpr (DBG & 8) dbg_t1 = dbg_stamp<DBG>();
+    QGEMM_STAMP(1);
     if constexpr (C::PIPE != PIPE_SIMPLE) {
         // (ping-pong) Waves 4-7 ("late" group) run one phase behind waves 0-3 ("early" group).  Phases:
         //   memory : ds_read all fragments of tile kt into registers
@@ -552,7 +535,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             }
         };
         auto issue_a1 = [&](int i, int kt, int buf) {
-            if constexpr (DBG & 2) return;
             if constexpr (VOFF_PER_COPY) {
                 char *grp = smem + buf * C::A_BYTES + (wave * LPT_A + (i & ~3)) * 1024;
                 dma(ra_g, grp, vo_copy[i], (uint32_t)kt * C::BKB, i & 3);
@@ -562,7 +544,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             }
         };
         auto issue_b1 = [&](int i, int kt) {
-            if constexpr (DBG & 2) return;
             if constexpr (VOFF_PER_COPY) {
                 const int il = i - LPT_A;
                 char *grp = smem + B_BASE + (kt & 1) * C::B_BYTES + (wave * LPT_B + (il & ~3)) * 1024;
@@ -614,7 +595,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             v2i as_pair[NLD];
             constexpr bool as_kcont = C::ASK;
             auto fetch_a_scales = [&](int kt, int comp) {      // for K step kt (of this slice; comp = kt & 1)
-                if constexpr (C::BLOCK_SCALE && !(DBG & 256)) {
+                if constexpr (C::BLOCK_SCALE) {
                     const uint32_t kb = kbeg + kt;
                     if (as_kcont) {
                         if (comp == 0) {
@@ -631,7 +612,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 }
             };
             auto fetch_b_scales = [&](int kt) {
-                if constexpr (C::BLOCK_SCALE && !(DBG & 256)) {
+                if constexpr (C::BLOCK_SCALE) {
                     // (one step past the end of K is fetched like the others: keep that read inside the array)
                     const uint32_t kb = kbeg + kt, kbc = kb < p.ksteps ? kb : p.ksteps - 1;
 #pragma unroll
@@ -644,8 +625,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
                     for (int j = 0; j < NLD; ++j) {
-                        unsigned x = (DBG & 256) ? __builtin_bit_cast(unsigned, 1.0f) : (unsigned)as_pair[j][comp];
-                        if constexpr (NBS == 1 && !(DBG & 256))
+                        unsigned x = (unsigned)as_pair[j][comp];
+                        if constexpr (NBS == 1)
                             x = __builtin_bit_cast(unsigned, __builtin_bit_cast(float, x) * bs_raw[0]);
                         const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);      // (R0 R0 R2 R2), (R1 R1 R3 R3)
                         const auto e = __builtin_amdgcn_permlane32_swap(r[0], r[0], false, false);  // all R0, all R2
@@ -660,13 +641,11 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 }
             };
             auto rd_a = [&](int buf, int a, int slot) {
-                if constexpr (DBG & 4) return;
                 const char *sa_ = smem + buf * C::A_BYTES;
                 far[slot][0] = frag_a(sa_, a, 0);
                 far[slot][1] = frag_a(sa_, a, 1);
             };
             auto rd_b = [&](int kt, int b) {
-                if constexpr (DBG & 4) return;
                 const char *sb_ = smem + B_BASE + (kt & 1) * C::B_BYTES - C::A_BYTES;   // frag_b adds RBA row blocks
                 fbr[b][0] = frag_b(sb_, b, 0);
                 fbr[b][1] = frag_b(sb_, b, 1);
@@ -676,7 +655,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             constexpr bool PINNED = C::NW == 4;
             constexpr int HALVES = (PINNED && C::ARITH != AR_F8) ? 2 : 1;
             auto mma = [&](int a, int b, int half) {
-                if constexpr (DBG & 1) return;
                 if constexpr (PINNED)
                     mma128_inplace<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1], acc[a][b], half);
                 else
@@ -700,7 +678,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 fetch_a_scales(kt + 1, par ^ 1);
                 fetch_b_scales(kt + 1);
                 auto fold = [&](int i) {
-                    if constexpr (C::BLOCK_SCALE && !(DBG & 1) && !(DBG & 128)) {
+                    if constexpr (C::BLOCK_SCALE) {
                         const int pa = i / C::TN, pb = i % C::TN;
                         const float f = sc[pa % 2][(pb * 16) / 128];
 #pragma unroll
@@ -709,7 +687,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 };
 #pragma unroll
                 for (int a = 0; a < TMs; ++a) {
-                    if (a == BR && !(DBG & 64)) {
+                    if (a == BR) {
                         __builtin_amdgcn_sched_barrier(0);
                         // lgkmcnt(0) and vmcnt(LPT_A): all but the A copies of this step
                         __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A) & 0xF0FF);
@@ -719,7 +697,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     // of the row would leave the matrix core idle once they take longer than one MFMA
                     auto side = [&](int slot) {      // slot 0 .. TN-1: what rides behind MFMA `slot` of this row
                         if (slot < 2) {              // the two halves of the A fragment AHEAD rows ahead
-                            if constexpr (DBG & 4) return;
                             const int an = a + AHEAD;
                             const int buf = an < TMs ? a_rd : a_nx, ar = an < TMs ? an : an - TMs;
                             far[an % RING][slot] = frag_a(smem + buf * C::A_BYTES, ar, slot);
@@ -744,9 +721,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #pragma unroll
                         for (int b = 0; b < C::TN; ++b) {
                             const int i = a * C::TN + b;
-                            if constexpr (!(DBG & 1))
-                                part[i % (BEHIND + 1)] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0],
-                                                               far[a % RING][1], v4f{0, 0, 0, 0});
+                            part[i % (BEHIND + 1)] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1],
+                                                                      v4f{0, 0, 0, 0});
                             side(b);
                             if (b == 1) {        // factor of this row, first used behind the next MFMA
 #pragma unroll
@@ -775,7 +751,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                                 // each half as soon as its MFMA of the last row is out, so the first halves, which
                                 // the next step needs first, are read half a row earlier)
                                 if constexpr (HALVES == 2) {
-                                    if (a == TMs - 1 && !(DBG & 4)) {
+                                    if (a == TMs - 1) {
                                         const char *sb_ = smem + B_BASE + ((kt + 1) & 1) * C::B_BYTES - C::A_BYTES;
                                         fbr[b][h] = frag_b(sb_, b, h);
                                     }
@@ -857,14 +833,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             int a_rd = 0;                       // buffer holding A of the tile being read
             // kt: tile the early group reads in this slot; guard: check the end of K
             auto issue_even = [&](int j, int kt, bool guard) {
-                if constexpr (DBG & 2) return;
                 if (guard && kt + 1 >= nk) return;
                 if constexpr (C::A3) issue_b1(LPT_A + j, kt + 1);
                 else if (j < LPT_A) issue_a1(j, kt + 1, a_wr);
                 else issue_b1(j, kt + 1);
             };
             auto issue_odd = [&](int j, int kt, bool guard) {
-                if constexpr (DBG & 2) return;
                 if constexpr (C::A3) {
                     if (guard && kt + 2 >= nk) return;
                     issue_a1(j, kt + 2, a_wr);
@@ -872,17 +846,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             };
             v4i fa[C::TM][2], fb[C::TN][2];
             constexpr int COLS_COPY = C::TN - C::TAIL;    // copies that can ride between the MFMA columns
-
-            // DBG bit 4: accumulate cycles per phase section (s_memtime, so only taken at points
-            // where no LDS read is outstanding)
-            unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, tprev = 0;
-            auto stamp = [&](int slot) {
-                if constexpr (DBG & 16) {
-                    const unsigned long long t = __builtin_readcyclecounter();
-                    ph[slot] += t - tprev;
-                    tprev = t;
-                }
-            };
 
             // one K step of one wave.  LATE / GUARD are std::integral_constant<bool>.
             auto step = [&](int kt, auto late_tag, auto guard_tag) {
@@ -895,39 +858,34 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 const char *sa_ = smem + a_rd * C::A_BYTES;
                 const char *sb_ = smem + B_BASE + (kt & 1) * C::B_BYTES - C::A_BYTES;   // frag_b adds RBA row blocks
                 constexpr int n_m = LATE ? N_ODD : N_EVEN;     // copies of this wave in this phase
-                if (!(DBG & 4) || kt == 0) {
     #pragma unroll
-                    for (int a = 0; a < C::TM; ++a) {
-                        if (a < n_m) {
-                            if constexpr (LATE) issue_odd(a, kt, GUARD);
-                            else issue_even(a, kt, GUARD);
-                        }
-                        fa[a][0] = frag_a(sa_, a, 0);
-                        fa[a][1] = frag_a(sa_, a, 1);
+                for (int a = 0; a < C::TM; ++a) {
+                    if (a < n_m) {
+                        if constexpr (LATE) issue_odd(a, kt, GUARD);
+                        else issue_even(a, kt, GUARD);
                     }
+                    fa[a][0] = frag_a(sa_, a, 0);
+                    fa[a][1] = frag_a(sa_, a, 1);
+                }
     #pragma unroll
-                    for (int b = 0; b < C::TN; ++b) {
-                        if (C::TM + b < n_m) {
-                            if constexpr (LATE) issue_odd(C::TM + b, kt, GUARD);
-                            else issue_even(C::TM + b, kt, GUARD);
-                        }
-                        fb[b][0] = frag_b(sb_, b, 0);
-                        fb[b][1] = frag_b(sb_, b, 1);
+                for (int b = 0; b < C::TN; ++b) {
+                    if (C::TM + b < n_m) {
+                        if constexpr (LATE) issue_odd(C::TM + b, kt, GUARD);
+                        else issue_even(C::TM + b, kt, GUARD);
                     }
+                    fb[b][0] = frag_b(sb_, b, 0);
+                    fb[b][1] = frag_b(sb_, b, 1);
                 }
                 if constexpr (LATE ? (N_ODD > 0) : !C::A3) a_wr = next_buf(a_wr);
                 a_rd = next_buf(a_rd);
                 __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());   // reads done before the buffers may be refilled
-                stamp(0);
                 auto wait_copies = [&]() {   // end of an odd slot: all copies landed but (A3) the A copy just issued
                     __builtin_amdgcn_sched_barrier(0);   // stays behind the MFMAs of the phase
                     if (C::A3 && (!GUARD || kt + 2 < nk)) __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
                     else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
                 };
                 if constexpr (LATE) wait_copies();
-                stamp(1);
                 phase_barrier();
-                stamp(2);
                 // ---- compute phase (early: slot 2kt+1, odd; late: slot 2kt+2, even)
                 constexpr int n_c = LATE ? N_EVEN : N_ODD;
                 const int kt_slot = LATE ? kt + 1 : kt;
@@ -958,18 +916,14 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                                     if constexpr (LATE) issue_even(b, kt_slot, GUARD);
                                     else issue_odd(b, kt_slot, GUARD);
                                 }
-                                if constexpr (!(DBG & 1))
-                                    part[i & 1] =
-                                        mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                                part[i & 1] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
                             }
                             __builtin_amdgcn_sched_barrier(0);   // MFMA i first, the FMAs of tile i-1 under it
                             if (i > b0 * C::TM) {
                                 const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
                                 const float f = sc[pa][(pb * 16) / 128];
-                                if constexpr (!(DBG & 1)) {
     #pragma unroll
-                                    for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f;
-                                }
+                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f;
                             }
                             __builtin_amdgcn_sched_barrier(0);
                         }
@@ -982,7 +936,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                             else issue_odd(b, kt_slot, GUARD);
                             __builtin_amdgcn_sched_barrier(0);
                         }
-                        if constexpr (DBG & 1) continue;
     #pragma unroll
                         for (int a = 0; a < C::TM; ++a)
                             acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
@@ -990,11 +943,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 };
                 mfma_cols(0, C::TN - C::TAIL, n_c < COLS_COPY ? n_c : COLS_COPY);
                 if constexpr (LATE ? !C::A3 : (N_ODD > 0)) a_wr = next_buf(a_wr);
-                stamp(3);
                 if constexpr (!LATE) wait_copies();
-                stamp(4);
                 if (!LATE || !GUARD || kt + 1 < nk) phase_barrier();
-                stamp(5);
                 mfma_cols(C::TN - C::TAIL, C::TN, 0);
             };
 
@@ -1023,19 +973,13 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     if (!C::A3) a_wr = next_buf(a_wr);
                     phase_barrier();
                 }
-                if constexpr (DBG & 16) tprev = __builtin_readcyclecounter();
                 int kt = 0;
                 for (; kt < nk_fast; ++kt) step(kt, yes_t{}, no_t{});
                 for (; kt < nk; ++kt) step(kt, yes_t{}, yes_t{});
             } else {
-                if constexpr (DBG & 16) tprev = __builtin_readcyclecounter();
                 int kt = 0;
                 for (; kt < nk_fast; ++kt) step(kt, no_t{}, no_t{});
                 for (; kt < nk; ++kt) step(kt, no_t{}, yes_t{});
-            }
-            if constexpr (DBG & 16) {
-                if (lane == 0)
-                    for (int i = 0; i < 6; ++i) p.dbg_cycles[((size_t)blockIdx.x * C::NW + wave) * 8 + i] = ph[i];
             }
         }
     } else {
@@ -1208,7 +1152,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     }
 
-    if constexpr (DBG & 8) dbg_t2 = dbg_stamp<DBG>();
+    QGEMM_STAMP(2);
     // ---- epilogue: lane holds C[m][n0 .. n0+3] of every 16x16 tile
     float scale = 1.0f;
     if (p.per_matrix_scale) scale = p.as[0] * p.bs[0];
@@ -1353,13 +1297,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
       };
       if (DT == QGEMM_DT_BF16 || DT == QGEMM_DT_F16) run(std::integral_constant<int, 2>{});
       else run(std::integral_constant<int, 4>{});
-        if constexpr (DBG & 8) {
-            const unsigned long long t3 = dbg_stamp<DBG>();
-            if (lane == 0 && !(DBG & 16)) {
-                unsigned long long *o = p.dbg_cycles + ((size_t)blockIdx.x * C::NW + wave) * 4;
-                o[0] = dbg_t0; o[1] = dbg_t1; o[2] = dbg_t2; o[3] = t3;
-            }
-        }
+        QGEMM_STAMP(3);
+        QGEMM_STAMP_WRITE(p.dbg_cycles, blockIdx.x * C::NW + wave, 4, lane == 0);
         return;
     }
 #pragma unroll
@@ -1404,13 +1343,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             }
         }
     }
-    if constexpr (DBG & 8) {
-        const unsigned long long t3 = dbg_stamp<DBG>();
-        if (lane == 0) {
-            unsigned long long *o = p.dbg_cycles + ((size_t)blockIdx.x * C::NW + wave) * 4;
-            if constexpr (!(DBG & 16)) { o[0] = dbg_t0; o[1] = dbg_t1; o[2] = dbg_t2; o[3] = t3; }
-        }
-    }
+    QGEMM_STAMP(3);
+    QGEMM_STAMP_WRITE(p.dbg_cycles, blockIdx.x * C::NW + wave, 4, lane == 0);
 #endif
 }
 
