@@ -179,6 +179,56 @@ def vendor_sweep(Q, torch, dev):
     return rows
 
 
+def skinny_probe(Q, torch, dev):
+    """Where a launch of the skinny-M kernel spends its time (config 5 shapes, fp8):
+      * graph-replay time per launch with B resident against the number of 32-column strips (= workgroups), K and
+        M unchanged: tells a limit inside a CU from one in the L2 / fabric;
+      * with the measurement build of the library (QGEMM_LIBRARY=qgemm_amd/libqgemm_dbg.so, `make DEBUG=1`): the
+        kernel's own time stamps (100 MHz clock shared by all CUs), means over all waves of eager launches."""
+    K = 2048
+    out = {"resident_us_by_strips": {}, "stamps_ns": {}}
+    for M in (16, 64, 128):
+        a, sa = _quant_fp8(torch.randn(M, K, device=dev))
+        for N in (896, 1792, 3584, 7168):
+            b, sb = _quant_fp8(torch.randn(N, K, device=dev))
+            c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            us = _graph_time([lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX, split_k=1)] * 24)
+            out["resident_us_by_strips"]["M%d_strips%d" % (M, N // 32)] = round(us, 2)
+    try:
+        Q.set_option("dbg_ptr", 0)
+    except Q.QgemmError:
+        out["stamps_ns"] = "needs the measurement build: QGEMM_LIBRARY=qgemm_amd/libqgemm_dbg.so"
+        return out
+    N, NS, nbuf = 7168, 6, 24
+    buf = torch.zeros(224 * 8 * NS, dtype=torch.int64, device=dev)
+    Q.set_option("dbg_ptr", buf.data_ptr())
+    bs = [_quant_fp8(torch.randn(N, K, device=dev)) for _ in range(nbuf)]
+    names = ("wave_start", "copies_issued", "unused", "k_loop_done", "past_barrier", "kernel_end")
+    for M in (16, 64, 128):
+        a, sa = _quant_fp8(torch.randn(M, K, device=dev))
+        c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        for mode in ("rotated", "resident"):
+            acc, last = None, 0.0
+            for r in range(30):
+                b, sb = bs[r % nbuf] if mode == "rotated" else bs[0]
+                buf.zero_()
+                torch.cuda.synchronize()
+                Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)
+                torch.cuda.synchronize()
+                if r < 6:
+                    continue
+                t = buf.view(224 * 8, NS).double() * 10.0             # 100 MHz ticks -> ns
+                rel = t - t[:, 0].min()
+                row = rel.mean(dim=0)
+                acc = row if acc is None else acc + row
+                last += float(rel[:, 5].max())
+            acc /= 24
+            out["stamps_ns"]["M%d_%s" % (M, mode)] = dict(
+                {n: round(float(v)) for n, v in zip(names, acc.tolist()) if n != "unused"}, last_wave_end=round(last / 24))
+    Q.set_option("dbg_ptr", 0)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -196,6 +246,8 @@ def main():
     ap.add_argument("--vendor-sweep", action="store_true",
                     help="only time this library against the vendor library (torch.matmul, torch._scaled_mm, "
                          "torch._int_mm) over a list of shapes, interleaved, print one JSON line and exit")
+    ap.add_argument("--skinny-probe", action="store_true",
+                    help="only probe where the skinny-M kernel (config 5) spends its time, print one JSON line and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists).", file=sys.stderr)
@@ -219,6 +271,9 @@ def main():
     dev = "cuda:0"
     if args.vendor_sweep:
         print(json.dumps({"vendor_sweep": vendor_sweep(Q, torch, dev)}))
+        return 0
+    if args.skinny_probe:
+        print(json.dumps({"skinny_probe": skinny_probe(Q, torch, dev)}))
         return 0
     M = N = K = args.size
 
