@@ -60,6 +60,7 @@ struct Context {
 #if QGEMM_DEBUG_BUILD
     long dbg_ptr = 0;           // measurement builds: device buffer for the kernels' time stamps (GemmArgs::dbg_cycles)
 #endif
+    long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes
     std::string last_config;
@@ -540,6 +541,10 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
         const int vec = ob == 4 ? 16 : 8;
         a.vec_store = ((uintptr_t)q.C % vec == 0) && ((q.ldc * ob) % vec == 0);
         if (a.vec_store && (uintptr_t)q.C % 16 == 0 && (q.ldc * ob) % 16 == 0) a.vec_store = 2;
+        // 4-byte C over at least three rounds of 256 x 256 tiles: spread the write bursts (see gemm_nt_kernel)
+        const bool spread = v.bm == 256 && v.bn == 256 && ob == 4 && pl.tiles >= 3 * (size_t)g_ctx.num_cus;
+        a.stagger = g_ctx.stagger >= 0 ? (uint32_t)g_ctx.stagger : (spread ? 2u : 0u);
+        a.stagger_wgs = (uint32_t)g_ctx.num_cus;
         hipError_t e = v.launch(a, (uint32_t)pl.tiles, stream);
         g_ctx.last_config = std::string(v.name) + kmaj_suffix(q.kmaj);
         return e == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
@@ -786,6 +791,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "force_split")) g_ctx.force_split = value;
     else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
     else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
+    else if (!std::strcmp(key, "stagger")) g_ctx.stagger = value;
 #if QGEMM_DEBUG_BUILD
     else if (!std::strcmp(key, "dbg_ptr")) g_ctx.dbg_ptr = value;
 #endif
