@@ -1203,15 +1203,19 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     } else if constexpr (C::PIPE == PIPE_SIMPLE && EPI_FITS) {
         __syncthreads();
     }
-    const bool wave_tile_full = row0 + wm * C::WM + C::WM <= p.M && col0 + wn * C::WN + C::WN <= p.N;
+    // columns of the wave tile inside C; rows of it inside C (at most WM; none or fewer where the tile sticks out below)
+    const bool wave_cols_full = col0 + wn * C::WN + C::WN <= p.N;
+    const int wave_rows = (int)p.M - (int)(row0 + wm * C::WM);
     // Every accumulator is read in exactly one place (write_slab): the output type is a uniform branch around
-    // the conversion of a slab, and wave tiles that stick out of C or meet unaligned rows take the same way
-    // through the scratch and differ only in how a slab leaves it (element by element, bounds checked).
+    // the conversion of a slab, and wave tiles that stick out of C sideways or meet unaligned rows take the same way
+    // through the scratch and differ only in how a slab leaves it (element by element, bounds checked).  A wave tile
+    // that sticks out below C (M is whatever the caller's batch is; N and the alignment come with the weights)
+    // keeps the 16-byte stores and leaves out the rows past M; so does one that sticks out sideways when the rows of C
+    // end on a 16-byte boundary (its lanes past N leave their pieces out).
     // With the accumulators of a 128 x 128 wave tile pinned in the 256 accumulation registers, several code
     // paths that each name all of them made the register allocator spill two dozen of them to memory here.
     if constexpr (EPI_FITS) {
       const int DT = p.out_dtype;
-      const bool fast = p.vec_store == 2 && wave_tile_full;
       // the element size of the output is a compile-time constant of the slab code (two copies of it: the
       // addressing of the scratch depends on it); the type of that size is a uniform branch inside
       auto run = [&](auto es_tag) {
@@ -1228,6 +1232,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         const int wr_off = (lane & 15) * PITCH + (lane >> 4) * 4 * ES;
         const size_t c_row_bytes = (size_t)p.ldc * ES;
         const uint32_t wrow0 = row0 + wm * C::WM, wcol0 = col0 + wn * C::WN;
+        // 16-byte stores: C and its rows aligned, and every 16-byte piece of a row either inside C or outside
+        const bool fast = p.vec_store == 2 && (wave_cols_full || ((size_t)p.N * ES) % 16 == 0);
+        const bool lane_in_cols = rd_col < ((int)p.N - (int)wcol0) * ES;
         char *cwave = Cz + ((size_t)wrow0 * p.ldc + wcol0) * ES;
         // Accumulators pinned in the accumulation registers (4-wave solo pipeline) are fetched from there one
         // slab at a time; left to itself the compiler moves all 256 of them into vector registers first.
@@ -1289,8 +1296,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 if (a + 1 < C::TM) write_slab(a + 1);
 #pragma unroll
                 for (int ps = 0; ps < PASSES; ++ps)
-                    __builtin_nontemporal_store(
-                        v[ps], (v4i *)(cwave + rd_col + (size_t)(a * 16 + rd_row + ps * RPP) * c_row_bytes));
+                    if (lane_in_cols && a * 16 + rd_row + ps * RPP < wave_rows)
+                        __builtin_nontemporal_store(
+                            v[ps], (v4i *)(cwave + rd_col + (size_t)(a * 16 + rd_row + ps * RPP) * c_row_bytes));
             } else {
                 if (a + 1 < C::TM) write_slab(a + 1);
                 // any alignment, any overhang: one element per lane and turn

@@ -1,6 +1,7 @@
 """Leading dimensions on the MFMA path: ldC > N (the one stride the reference honours,
 src/gemm/sm89_gemm_kernel_v3.cu:258), ldA > K and ldB > K, through every way a tile leaves the kernel
-(16-byte row pieces, element by element from a ragged or unaligned tile, the tiles without LDS staging),
+(16-byte row pieces from whole and from ragged tiles, element by element from an unaligned tile, the tiles without
+LDS staging),
 with and without a K split.  The padding columns of C and a guard row behind it are filled with a poison
 value that has to survive."""
 import numpy as np
@@ -39,7 +40,8 @@ EXITS = [2, 11, 12, 13, 15, 16]
 
 @pytest.mark.parametrize("pad", [8, 5])
 @pytest.mark.parametrize("variant", EXITS)
-@pytest.mark.parametrize("shape", [(256, 512, 256), (300, 333, 256)])      # whole wave tiles / ragged
+# whole wave tiles / ragged / ragged with rows that end on a 16-byte boundary (16-byte stores, rows and lanes left out)
+@pytest.mark.parametrize("shape", [(256, 512, 256), (300, 333, 256), (300, 328, 256)])
 @pytest.mark.parametrize("split", [1, 2])
 def test_int8_padded_ldc(pad, variant, shape, split):
     M, N, K = shape
@@ -56,7 +58,7 @@ def test_int8_padded_ldc(pad, variant, shape, split):
 
 @pytest.mark.parametrize("pad", [8, 5])
 @pytest.mark.parametrize("variant", EXITS)
-@pytest.mark.parametrize("shape", [(256, 512, 256), (300, 333, 256)])
+@pytest.mark.parametrize("shape", [(256, 512, 256), (300, 333, 256), (300, 328, 256)])
 def test_fp8_bf16_out_padded_ldc(pad, variant, shape):
     M, N, K = shape
     say("ldC fp8 -> bf16", shape, "pad", pad, "variant", variant)
