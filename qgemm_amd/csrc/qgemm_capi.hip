@@ -406,21 +406,30 @@ struct Plan {
     std::unique_ptr<Plan> rest;
 };
 
-// Rows of the problem that the 256 x 256 tile should keep when its tiles do not fill the last round of CUs.
-// 576 tiles on 256 CUs are 2.25 rounds and cost three: the rows of the two full rounds stay, and the rows below
-// go to whatever the estimate likes best for them (smaller tiles, which fill the CUs).  Returns 0 for "do not
-// split": when the estimate of the two launches (plus 6 us for the second) is not at least 3 % below the one.
-size_t rows_for_full_rounds(const Variant *tab, int count, const Variant &v, size_t M, size_t N, size_t ksteps, bool block,
-                            int cus, double t_single) {
-    if (v.bm != 256 || v.bn != 256 || !g_ctx.row_split) return 0;
+// Rows of the problem that 256 x 256 tiles should take when such tiles do not fill the last round of CUs.
+// 576 tiles on 256 CUs are 2.25 rounds and cost three: the rows of the two full rounds go to one launch, and the
+// rows below to whatever the tile choice likes best for them (smaller tiles, which fill the CUs; the skinny-M
+// kernel for up to 128 rows).  Also where a single launch would rather take smaller tiles for everything
+// (5000 x 4096 x 7168: 1.25 rounds of 256 x 256 tiles; fp8 148 us as one launch of 128 x 128 tiles, 113 us as 4096 rows
+// of 256 x 256 tiles and 904 rows of 128 x 128 ones; 7000 x 7168 x 2048: 106 -> 93 us with the last 88 rows on the
+// skinny-M kernel).  Returns 0 for "do not split": when the estimate of the two launches (plus 6 us for the
+// second) is not at least 3 % below the estimate t_single of the one.
+size_t rows_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus,
+                            double t_single) {
+    if (!g_ctx.row_split) return 0;
     const size_t tn = (N + 255) / 256, tiles = ((M + 255) / 256) * tn, full = tiles / cus;
     if (full == 0 || tiles % cus == 0) return 0;
     const size_t m_main = (full * cus / tn) * 256;
-    if (m_main == 0 || m_main + 128 >= M) return 0;          // (the estimate is for more than 128 rows)
+    if (m_main == 0 || m_main >= M) return 0;
     uint32_t ns = 0;
     double t_main = 0, t_rest = 0;
-    if (choose_by_cost(tab, count, m_main, N, ksteps, block, cus, false, &ns, &t_main) < 0) return 0;
-    if (choose_by_cost(tab, count, M - m_main, N, ksteps, block, cus, false, &ns, &t_rest) < 0) return 0;
+    const int vm = choose_by_cost(tab, count, m_main, N, ksteps, block, cus, false, &ns, &t_main);
+    if (vm < 0 || tab[vm].bm != 256 || tab[vm].bn != 256) return 0;
+    if (M - m_main > 128) {
+        if (choose_by_cost(tab, count, M - m_main, N, ksteps, block, cus, false, &ns, &t_rest) < 0) return 0;
+    } else {
+        t_rest = 5.0 + (double)N * ksteps * 128.0 / 4.0e6;      // B streamed once, about 4 TB/s
+    }
     return t_main + t_rest + 6.0 < 0.97 * t_single ? m_main : 0;
 }
 
@@ -436,7 +445,7 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
         double t_single = 0;
         const int ci = choose_by_cost(tab, count, q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, false, &ns, &t_single);
         if (ci >= 0 && tab[ci].bm == tab[vi].bm && tab[ci].bn == tab[vi].bn && tab[ci].kgroups == tab[vi].kgroups) {
-            const size_t m_main = rows_for_full_rounds(tab, count, tab[vi], q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, t_single);
+            const size_t m_main = rows_for_full_rounds(tab, count, q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, t_single);
             if (m_main) {
                 NtProblem q_main = q, q_rest = q;
                 q_main.M = m_main;
@@ -542,7 +551,9 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
         a.vec_store = ((uintptr_t)q.C % vec == 0) && ((q.ldc * ob) % vec == 0);
         if (a.vec_store && (uintptr_t)q.C % 16 == 0 && (q.ldc * ob) % 16 == 0) a.vec_store = 2;
         // 4-byte C over at least three rounds of 256 x 256 tiles: spread the write bursts (see gemm_nt_kernel)
-        const bool spread = v.bm == 256 && v.bn == 256 && ob == 4 && pl.tiles >= 3 * (size_t)g_ctx.num_cus;
+        // (with fewer than 32 K steps the offsets are too large a part of a tile's time: 7000 x 7168 x 2048 int8 to
+        // f32 128 us without, 139 us with)
+        const bool spread = v.bm == 256 && v.bn == 256 && ob == 4 && pl.tiles >= 3 * (size_t)g_ctx.num_cus && a.ksteps >= 32;
         a.stagger = g_ctx.stagger >= 0 ? (uint32_t)g_ctx.stagger : (spread ? 2u : 0u);
         a.stagger_wgs = (uint32_t)g_ctx.num_cus;
         hipError_t e = v.launch(a, (uint32_t)pl.tiles, stream);

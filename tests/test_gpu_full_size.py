@@ -206,3 +206,40 @@ def test_row_split_of_a_partly_empty_last_round():
     name = Q.last_config()
     assert "+" in name, name
     assert_close(host(c16)[rows], R.gemm_f32acc(R.decode_bf16(ha[rows]), R.decode_bf16(hb)), rtol=1e-4, atol=1e-3, what=name)
+
+
+@pytest.mark.parametrize("shape,m_main,rest", [((4184, 4096, 2048), 4096, "skinny_128x32_k8"),     # 88 rows below one full round
+                                               ((5000, 4096, 2048), 4096, "128x128")])            # single launch: 128 x 128 tiles
+def test_row_split_with_a_short_rest_and_against_smaller_tiles(shape, m_main, rest):
+    """Row split where the rows below the full rounds are at most 128 (they go to the skinny-M kernel) and where a
+    single launch would have taken smaller tiles for everything.  int8: the integers of the single launch
+    everywhere and the oracle's on rows of both parts and at the seam; fp8 per-matrix to bf16: the oracle within
+    tolerance on the same rows."""
+    M, N, K = shape
+    say("row split", shape)
+    plan = Q.plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, M, N, K)
+    assert plan.startswith("256x256") and "+" in plan and rest in plan.split("+")[1], plan
+    rng = np.random.default_rng(77)
+    qa = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    qb = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    da, db_ = dev(qa), dev(qb)
+    c = torch.full((M, N), -5, dtype=torch.int32, device="cuda")
+    Q.int8_mm(da, db_, scalar(1.0), scalar(1.0), c)
+    name = Q.last_config()
+    assert name == plan, (name, plan)
+    rows = np.concatenate([_sample(m_main, 10, 5), m_main + _sample(M - m_main, 10, 6), [m_main - 1, m_main, M - 1]])
+    assert np.array_equal(host(c)[rows], R.gemm_i8_i32(qa[rows], qb)), name
+    Q.set_option("row_split", 0)
+    c1 = torch.full((M, N), -6, dtype=torch.int32, device="cuda")
+    Q.int8_mm(da, db_, scalar(1.0), scalar(1.0), c1)
+    assert "+" not in Q.last_config() and torch.equal(c, c1)
+    Q.set_option("row_split", 1)
+
+    qa8, sa = R.quantize_fp8(R.fill_normal((M, K), 51))
+    qb8, sb = R.quantize_fp8(R.fill_normal((N, K), 52))
+    cb = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa8), fp8_tensor(qb8), scalar(sa), scalar(sb), cb, M, N, K, Q.SCALE_PER_MATRIX)
+    name = Q.last_config()
+    assert "+" in name, name
+    ref = R.gemm_f32acc(R.decode_fp8(qa8[rows]), R.decode_fp8(qb8)) * np.float32(sa * sb)
+    assert_close(host(cb)[rows], ref, what=name)
