@@ -586,7 +586,15 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
     r.part_is_i32 = i32_acc;
     r.out_dtype = q.out_dtype;
     r.per_matrix_scale = q.per_matrix;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((plane + 255) / 256)), dim3(256), 0, stream, r);
+    if (q.N % 4 == 0) {
+        const int ob = dtype_bytes(q.out_dtype), c_align = ob == 4 ? 16 : 8;
+        const int c_vec = (uintptr_t)q.C % c_align == 0 && (q.ldc * ob) % c_align == 0;
+        const dim3 grid((unsigned)((plane / 4 + 255) / 256));
+        if (i32_acc) hipLaunchKernelGGL(splitk_reduce4_kernel<true>, grid, dim3(256), 0, stream, r, c_vec);
+        else hipLaunchKernelGGL(splitk_reduce4_kernel<false>, grid, dim3(256), 0, stream, r, c_vec);
+    } else {
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((plane + 255) / 256)), dim3(256), 0, stream, r);
+    }
     g_ctx.last_config = std::string(v.name) + kmaj_suffix(q.kmaj) + "_splitk" + std::to_string(a.nsplit);
     return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
 }
