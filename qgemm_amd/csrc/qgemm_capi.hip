@@ -246,8 +246,9 @@ bool mfma_shape_ok(const NtProblem &q) {
 // partial planes.  The times per 128-byte K step were read off a sweep of every variant over square and oblong
 // shapes from 1024 to 8192 (fp8 and bf16 agree per step; block scales cost about a third more): 1.25 us for the
 // 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.52 us for the 128 x 128
-// row with two K groups (one per CU: it only wins where there are no more tiles than CUs), 0.45 us for 64 x 128,
-// 0.36 us for 128 x 32.
+// row with two K groups (one per CU: it only wins where there are no more tiles than CUs), 0.52 us for 64 x 128 and
+// 0.40 us for its row with two K groups (graph replays of 384 / 512 x 4096 x 4096 and 1024 x 2048 x 7168), 0.39 us for
+// 128 x 32.  A K split adds 4 us and the partial planes at 3 TB/s.
 //
 // M <= 64 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
 // workgroup, else the shortest tile that covers the rows; narrow tiles instead of a K split.  (65 .. 128 rows go
@@ -259,8 +260,8 @@ struct TileModel {
     bool kgroups;                              // the row of this tile with two K groups per workgroup (GemmCfg::KG)
 };
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false}, {128, 128, 2, 0.85, 0.66, 2.0, false},
-                                 {128, 128, 1, 0.52, 0.52, 3.0, true},  {64, 128, 1, 0.45, 0.45, 1.5, false},
-                                 {64, 128, 1, 0.42, 0.42, 2.5, true},   {128, 32, 1, 0.36, 0.36, 1.0, false}};
+                                 {128, 128, 1, 0.52, 0.52, 3.0, true},  {64, 128, 1, 0.52, 0.52, 1.5, false},
+                                 {64, 128, 1, 0.40, 0.40, 2.5, true},   {128, 32, 1, 0.39, 0.39, 1.0, false}};
 // rows with two K groups: eight waves on a tile that otherwise has four (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 
