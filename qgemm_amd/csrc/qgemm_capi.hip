@@ -738,7 +738,13 @@ int quantize_t(int mode, QuantArgs &a, hipStream_t stream) {
     } else if (mode == QGEMM_QUANT_BLOCK_1x128) {
         const uint64_t nblocks = (uint64_t)a.rows * ((a.cols + 127) / 128);
         if ((nblocks + 7) / 8 >= ((uint64_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
-        hipLaunchKernelGGL(quant_row_block_kernel<IN_DT>, dim3((unsigned)((nblocks + 7) / 8)), dim3(256), 0, stream, a);
+        const uint32_t nbc = a.cols / 128;
+        const bool whole = a.cols % 128 == 0 && a.ld % 4 == 0 && (uintptr_t)a.x % 16 == 0 && a.ldq % 4 == 0 &&
+                           (uintptr_t)a.q % 4 == 0 && a.out_dtype == QGEMM_DT_F8E4M3 && (nbc + 7) / 8 <= 65535 && a.rows > 0;
+        if (whole)
+            hipLaunchKernelGGL(quant_row_block_whole_kernel<IN_DT>, dim3(a.rows, (nbc + 7) / 8), dim3(256), 0, stream, a);
+        else
+            hipLaunchKernelGGL(quant_row_block_kernel<IN_DT>, dim3((unsigned)((nblocks + 7) / 8)), dim3(256), 0, stream, a);
     } else {
         const uint64_t nblocks = (uint64_t)((a.rows + 127) / 128) * ((a.cols + 127) / 128);
         if (nblocks >= ((uint64_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;

@@ -117,3 +117,49 @@ def test_quantise_then_multiply_block_scaled():
     # the result only differs from a GEMM on the unquantised operands by the quantisation error
     exact = a.astype(np.float64) @ b.astype(np.float64).T
     assert np.abs(host(c) - exact).max() < 0.06 * np.abs(exact).max()
+
+
+def test_division_by_the_scale_is_the_ieee_division():
+    """The quantisers divide every element of a block by one scale and share the reciprocal's refinement between
+    the elements; the quotients have to be those of the IEEE division the oracle does, bit for bit after encoding.
+    Random mantissas over twelve octaves below the block maximum (ties of the e4m3 and int8 rounding are hit
+    through the sheer number: 4 M elements), blocks whose scale lies on both sides of the range the shared form
+    covers (2^-60 .. 2^60) and far outside, elements that make quotients below 2^-100, signed zeros, infinities
+    and NaNs of both signs."""
+    rng = np.random.default_rng(1234)
+    rows, cols = 2048, 2048
+    mant = rng.integers(0, 1 << 23, (rows, cols), dtype=np.uint32)
+    expo = rng.integers(115, 128, (rows, cols), dtype=np.uint32)          # 2^-12 .. 2^0
+    sign = rng.integers(0, 2, (rows, cols), dtype=np.uint32) << 31
+    x = (sign | (expo << 23) | mant).view(np.float32)
+    # per row a magnitude: the scales of the 1 x 128 blocks then run from far below 2^-60 to far above 2^60
+    row_exp = np.linspace(-100, 100, rows).round().astype(np.int32)
+    x = np.ldexp(x, row_exp[:, None]).astype(np.float32)
+    # specials sprinkled in: tiny elements (quotient < 2^-100), signed zeros, infinities, NaNs
+    x[:, 5] = np.ldexp(np.float32(1.5), row_exp - 120).astype(np.float32)
+    x[:, 6] = -x[:, 5]
+    x[:, 130] = 0.0
+    x[:, 131] = -0.0
+    x[::7, 300] = np.inf
+    x[::11, 301] = -np.inf
+    x[::5, 400] = np.nan
+    x[::9, 401] = np.float32(-np.nan)
+    say("quantize: division by the shared scale", x.shape)
+    for mode, br in ((Q.QUANT_BLOCK_1x128, 1), (Q.QUANT_BLOCK_128x128, 128)):
+        q, s = R.quantize_fp8_block(x, br, 128)
+        g, gs = Q.quantize(dev(x), torch.float8_e4m3fn, mode)
+        assert np.array_equal(host(gs).view(np.uint32), s.view(np.uint32)), mode
+        assert np.array_equal(_u8(g), q), mode
+    # per matrix: one scale for everything; slices of rows keep the scale inside and outside the range
+    for lo, hi in ((0, 64), (1000, 1064), (2000, 2048), (400, 420)):
+        part = np.ascontiguousarray(x[lo:hi])
+        part = np.where(np.isfinite(part), part, np.float32(0)).astype(np.float32) if lo != 1000 else part
+        q, s = R.quantize_fp8(part)
+        g, gs = Q.quantize(dev(part), torch.float8_e4m3fn, Q.QUANT_PER_MATRIX)
+        assert host(gs).view(np.uint32)[0] == np.array([s], np.float32).view(np.uint32)[0]
+        assert np.array_equal(_u8(g), q), (lo, hi)
+        part = np.where(np.isfinite(part), part, np.float32(0)).astype(np.float32)
+        qi, si = R.quantize_int8(part)
+        gi, gsi = Q.quantize(dev(part), torch.int8, Q.QUANT_PER_MATRIX)
+        assert host(gsi).view(np.uint32)[0] == np.array([si], np.float32).view(np.uint32)[0]
+        assert np.array_equal(host(gi), qi), (lo, hi)
