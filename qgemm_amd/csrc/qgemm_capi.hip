@@ -748,7 +748,13 @@ int quantize_t(int mode, QuantArgs &a, hipStream_t stream) {
     } else {
         const uint64_t nblocks = (uint64_t)((a.rows + 127) / 128) * ((a.cols + 127) / 128);
         if (nblocks >= ((uint64_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
-        hipLaunchKernelGGL(quant_square_block_kernel<IN_DT>, dim3((unsigned)nblocks), dim3(256), 0, stream, a);
+        const bool whole = a.cols % 128 == 0 && a.rows % 128 == 0 && a.rows > 0 && a.cols > 0 && a.ld % 4 == 0 &&
+                           (uintptr_t)a.x % 16 == 0 && a.ldq % 4 == 0 && (uintptr_t)a.q % 4 == 0 &&
+                           a.out_dtype == QGEMM_DT_F8E4M3 && a.rows / 128 <= 65535;
+        if (whole)
+            hipLaunchKernelGGL(quant_square_block_whole_kernel<IN_DT>, dim3(a.cols / 128, a.rows / 128), dim3(256), 0, stream, a);
+        else
+            hipLaunchKernelGGL(quant_square_block_kernel<IN_DT>, dim3((unsigned)nblocks), dim3(256), 0, stream, a);
     }
     return hipGetLastError() == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
 }

@@ -274,4 +274,33 @@ __global__ void __launch_bounds__(256) quant_square_block_kernel(const QuantArgs
     }
 }
 
+// ---- 128 x 128 blocks, whole blocks (rows and cols multiples of 128), x and q aligned for vector access, fp8 out:
+// as above without the bounds checks
+template <int IN_DT>
+__global__ void __launch_bounds__(256) quant_square_block_whole_kernel(const QuantArgs p) {
+    __shared__ float red[4];
+    const uint32_t ib = blockIdx.y, jb = blockIdx.x;
+    const uint32_t c = jb * 128 + (threadIdx.x & 31) * 4;
+    const uint32_t r0 = ib * 128 + (threadIdx.x >> 5);            // rows r0, r0 + 8, ...
+    const size_t x0 = (size_t)r0 * p.ld + c, q0 = (size_t)r0 * p.ldq + c;
+    v4f v[16];
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = load4_as_f32<IN_DT>(p.x, x0 + (size_t)i * 8 * p.ld, true, 4);
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) m = __builtin_fmaxf(m, abs_or_zero(v[i][e]));
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    const float amax = __builtin_fmaxf(__builtin_fmaxf(red[0], red[1]), __builtin_fmaxf(red[2], red[3]));
+    const float s = scale_of(amax, QGEMM_DT_F8E4M3);
+    if (threadIdx.x == 0) p.scales[(size_t)ib * p.scale_rs + (size_t)jb * p.scale_cs] = s;
+    const Divisor dv = make_divisor(s);
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        *(uint32_t *)((uint8_t *)p.q + q0 + (size_t)i * 8 * p.ldq) = quant4(v[i], dv, QGEMM_DT_F8E4M3);
+}
+
 }  // namespace qgemm
