@@ -46,7 +46,7 @@ static hipError_t launch_skinny(const GemmArgs &a, uint32_t grid, hipStream_t s)
 template <int TM>
 static Variant skinny_row(const char *name) {
     using C = SkinnyCfg<INST_ARITH, TM>;
-    return Variant{name, C::ARITH, false, C::BM, C::BN, C::THREADS, C::LDS_BYTES, LOAD_DMA, false, 8, false, &launch_skinny<C>};
+    return Variant{name, C::ARITH, false, C::BM, C::BN, C::THREADS, C::LDS_BYTES, LOAD_DMA, false, 8, false, false, &launch_skinny<C>};
 }
 
 #define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) != PIPE_SIMPLE, INST_KMAJ>
@@ -63,7 +63,7 @@ template <bool OK, class C, class Fallback>
 static Variant row_of(const char *name, bool auto_ok) {
     using P = std::conditional_t<OK, C, Fallback>;
     return Variant{OK ? name : "128x128_w2x2_dma", P::ARITH, P::BLOCK_SCALE, P::BM, P::BN, P::THREADS, P::LDS_BYTES,
-                   P::LOADER, OK && auto_ok, P::KG, P::ASK, &launch_variant<P>};
+                   P::LOADER, OK && auto_ok, P::KG, P::ASK, P::AS_ANY_STRIDE, &launch_variant<P>};
 }
 #define ROWP(NAME, BM, BN, WM_, WN_, LD, PP, AUTO) \
     row_of<kmajor_can(BM, BN, (WM_) * (WN_), PP), CFG(BM, BN, WM_, WN_, LD, PP), CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>(NAME, AUTO)

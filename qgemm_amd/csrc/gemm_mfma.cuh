@@ -105,6 +105,11 @@ struct GemmCfg {
     // arrangement of QGEMM_LAYOUT_K_CONTIGUOUS, instead of rows contiguous, a_scale[m + kb * as_ks].  A compile-time
     // choice: as a branch inside the K loop it cost the 8-wave kernel 758 spilled registers.
     static constexpr bool ASK = ASK_;
+    // The simple and ping-pong pipelines load one scale per lane and K step at a_scale[m * as_ms + kb * as_ks] with
+    // whatever strides they are given: rows-contiguous scales are one 256-byte request per 64 rows, K-contiguous
+    // ones 64 requests, which these tiles (a step of several hundred cycles per wave) can afford and which saves the
+    // launch that would copy the scales into the other order.
+    static constexpr bool AS_ANY_STRIDE = BLOCK_SCALE_ && PIPE_ != PIPE_SOLO;
     // STAGES (simple pipeline, DMA loader): number of LDS stages, 0 = chosen below.
     // KGROUPS = 2: the workgroup has two sets of WAVES_M x WAVES_N waves; all of them copy, set 0 computes the
     // even K steps and set 1 the odd ones of the same tile (one barrier per pair of steps), and the two partial
@@ -420,7 +425,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             const uint32_t kb = kbeg + kt;
 #pragma unroll
             for (int j = 0; j < NLD; ++j)
-                as_raw[j] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (64 * j + kb * p.as_ks) * 4, 0);
+                as_raw[j] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (64 * j * p.as_ms + kb * p.as_ks) * 4, 0);
             // (the solo pipeline fetches one step past the end of K: keep that read inside the array)
             const uint32_t kbc = kb < p.ksteps ? kb : p.ksteps - 1;
 #pragma unroll

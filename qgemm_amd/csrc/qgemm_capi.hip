@@ -626,12 +626,24 @@ bool settle_scale_layout(const NtProblem &q, Plan &pl) {
             if (tab[i].a_scale_k_contiguous == ks && want == tab[i].name) return &tab[i];
         return nullptr;
     };
-    bool ks = q.as_ms != 1 && q.as_ks == 1 && q.as_ms % 2 == 0 && ((uintptr_t)q.as & 7u) == 0;
-    for (const Plan *p = &pl; ks && p; p = p->rest.get())
-        ks = partner(p->v, true) && !(p->a.nsplit > 1 && p->a.ksteps_per_split % 2 != 0);
-    for (Plan *p = &pl; p; p = p->rest.get())
-        if (const Variant *v = partner(p->v, ks)) p->v = v;
-    return ks || q.as_ms == 1;
+    if (q.as_ms == 1) {                                  // rows-contiguous: every kernel but the twins reads that
+        for (Plan *p = &pl; p; p = p->rest.get())
+            if (const Variant *v = partner(p->v, false)) p->v = v;
+        return true;
+    }
+    // some other arrangement (K-contiguous, as QGEMM_LAYOUT_K_CONTIGUOUS passes it): fine where every launch of the
+    // plan either takes any strides (simple and ping-pong pipelines) or has a twin for it
+    const bool ks_form = q.as_ks == 1 && q.as_ms % 2 == 0 && ((uintptr_t)q.as & 7u) == 0;
+    bool as_is = true;
+    for (const Plan *p = &pl; as_is && p; p = p->rest.get()) {
+        if (p->v->a_scale_any_stride) continue;
+        as_is = ks_form && partner(p->v, true) && !(p->a.nsplit > 1 && p->a.ksteps_per_split % 2 != 0);
+    }
+    for (Plan *p = &pl; p; p = p->rest.get()) {
+        if (p->v->a_scale_any_stride) continue;
+        if (const Variant *v = partner(p->v, as_is)) p->v = v;
+    }
+    return as_is;
 }
 
 int scales_rows_contiguous(NtProblem &q, void *room, hipStream_t stream) {

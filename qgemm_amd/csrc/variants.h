@@ -17,6 +17,7 @@ struct Variant {
                     // 8: the skinny-M kernel, eight waves each computing every eighth K step (gemm_skinny.cuh)
     bool a_scale_k_contiguous;   // block scales: the kernel also reads a_scale[m * ld + kb] as the caller has it
                                  // (the others want it rows-contiguous, a_scale[m + kb * ld])
+    bool a_scale_any_stride;     // block scales: the kernel reads a_scale[m * ms + kb * ks] for any ms, ks
     hipError_t (*launch)(const GemmArgs &, uint32_t grid, hipStream_t);
 };
 
