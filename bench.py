@@ -381,6 +381,23 @@ def main():
                     "GBps_resident": nbytes / us_res / 1e3, "tflops": 2.0 * m5 * n5 * k5 / us_rot / 1e6,
                     "algorithmic_bytes": nbytes, "kernel": Q.last_config()}
             del b5s
+        # the same shapes with 128-block scales (the reference's FP8_GEMM_kernel arithmetic at decode-sized M): the
+        # skinny-M kernel with the fold in its K loop; bytes as above plus the scales
+        b5s = [_quant_fp8(torch.randn(n5, k5, device=dev))[0] for _ in range(nbuf)]
+        bs5 = torch.rand(n5 // 128, k5 // 128, device=dev) * 1.5 + 0.5
+        for m5 in (16, 64, 128):
+            a5, _ = _quant_fp8(torch.randn(m5, k5, device=dev))
+            as5 = torch.rand(m5, k5 // 128, device=dev) * 1.5 + 0.5
+            c5 = torch.empty(m5, n5, dtype=torch.bfloat16, device=dev)
+            mk = lambda bq: (lambda: Q.scaled_gemm(a5, bq, as5, bs5, c5, m5, n5, k5, Q.SCALE_BLOCK128))
+            us_rot = _graph_time([mk(bq) for bq in b5s])
+            us_res = _graph_time([mk(b5s[0])] * nbuf)
+            nbytes = n5 * k5 + m5 * k5 + m5 * n5 * 2 + as5.numel() * 4 + bs5.numel() * 4
+            extra["skinny_fp8_block_M%d" % m5] = {
+                "us_per_launch_rotated": us_rot, "us_per_launch_resident": us_res,
+                "GBps": nbytes / us_rot / 1e3, "frac_of_hbm_peak": nbytes / us_rot / 1e3 / PEAK_HBM_GBS,
+                "GBps_resident": nbytes / us_res / 1e3, "algorithmic_bytes": nbytes, "kernel": Q.last_config()}
+        del b5s
         # cfg 4 in the reference's own storage (A is K x M, B is K x N, scales [K/128, M] and [K/128, N/128])
         a4r, _ = _quant_fp8(torch.randn(k4, m4, device=dev))
         b4r, _ = _quant_fp8(torch.randn(k4, n4, device=dev))

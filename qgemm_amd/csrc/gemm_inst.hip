@@ -45,8 +45,9 @@ static hipError_t launch_skinny(const GemmArgs &a, uint32_t grid, hipStream_t s)
 // Picked by choose_variant in place of the narrow simple-pipeline tiles, never by the table scan (auto_ok = false).
 template <int TM>
 static Variant skinny_row(const char *name) {
-    using C = SkinnyCfg<INST_ARITH, TM>;
-    return Variant{name, C::ARITH, false, C::BM, C::BN, C::THREADS, C::LDS_BYTES, LOAD_DMA, false, 8, false, false, &launch_skinny<C>};
+    using C = SkinnyCfg<INST_ARITH, TM, (bool)INST_BLOCK>;
+    return Variant{name, C::ARITH, C::BLOCK_SCALE, C::BM, C::BN, C::THREADS, C::LDS_BYTES, LOAD_DMA, false, 8, false,
+                   C::BLOCK_SCALE, &launch_skinny<C>};
 }
 
 #define CFG(BM, BN, WM_, WN_, LD, PP) GemmCfg<INST_ARITH, (bool)INST_BLOCK, BM, BN, WM_, WN_, LD, PP, 0, (PP) != PIPE_SIMPLE, INST_KMAJ>
@@ -113,7 +114,7 @@ static const Variant kTable[] = {
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("64x128_w1x4_k2", true),
 #endif
     // skinny M (gemm_skinny.cuh): the K split inside the workgroup, no staging, no barrier in the K loop
-#if INST_BLOCK || INST_KMAJ      // (no block-scale or K-major form: aliases, so indices agree across families)
+#if INST_KMAJ      // (no K-major form: aliases, so indices agree across families)
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),

@@ -26,9 +26,16 @@
 
 namespace qgemm {
 
-template <int ARITH_, int TM_>
+template <int ARITH_, int TM_, bool BLOCK_SCALE_ = false>
 struct SkinnyCfg {
     static constexpr int ARITH = ARITH_;
+    // 128-block scales (fp8): every MFMA starts from zero and its product of one K block is folded into the running
+    // sum with a_scale[row, kb] * b_scale[strip, kb], as in gemm_nt_kernel.  The strip of 32 columns lies inside one
+    // 128-column block of b_scale.  a_scale is read with the caller's strides (lane l: row l of the tile, the rows of
+    // an MFMA tile picked out of that with ds_bpermute); the scales of a round are requested in front of the round's
+    // copies, so they have arrived wherever the copies they precede have.
+    static constexpr bool BLOCK_SCALE = BLOCK_SCALE_;
+    static_assert(!BLOCK_SCALE_ || ARITH_ == AR_F8, "block scales are defined for fp8 only");
     static constexpr int TM = TM_, TN = 2;                  // 16 x 16 MFMA tiles of the workgroup's tile
     static constexpr int BM = 16 * TM_, BN = 32;
     static constexpr int NW = 8, THREADS = NW * kWave;
@@ -125,12 +132,66 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     for (int a = 0; a < C::TM; ++a)
 #pragma unroll
         for (int b = 0; b < C::TN; ++b) acc[a][b] = acc_t{0, 0, 0, 0};
-    auto compute = [&](int s) {
+
+    // block scales of the two steps of the round in hand (cur) and of the round whose copies are on their way (nxt)
+    constexpr int NLD = C::BLOCK_SCALE ? (C::BM + 63) / 64 : 1;
+    int as_cur[2][NLD], as_nxt[2][NLD];
+    float bs_cur[2], bs_nxt[2];
+    __amdgpu_buffer_rsrc_t ras = make_rsrc(p.as, 0);
+    uint32_t as_voff = 0, bs_base = 0;
+    if constexpr (C::BLOCK_SCALE) {
+        ras = make_rsrc(p.as, ((p.ksteps - 1) * p.as_ks + (p.M - 1) * p.as_ms + 1) * 4);
+        as_voff = (row0 + lane) * p.as_ms * 4;
+        uint32_t nb = col0 / 128;
+        nb = nb < p.nb_max ? nb : p.nb_max;
+        bs_base = nb * p.bs_ns;
+    }
+    auto fetch_scales = [&](int k) {            // for steps k and k + 8 of this wave (called in front of their copies)
+        if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
-        for (int b = 0; b < C::TN; ++b)
+            for (int s = 0; s < 2; ++s) {
+                const uint32_t kb = kbeg + (uint32_t)(k + s * C::NW);
+                // (a step past the end of K multiplies zeros: any finite scale will do, so keep the reads inside)
+                const uint32_t kbc = kb < p.ksteps ? kb : p.ksteps - 1;
+#pragma unroll
+                for (int j = 0; j < NLD; ++j)
+                    as_nxt[s][j] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (64 * j * p.as_ms + kbc * p.as_ks) * 4, 0);
+                bs_nxt[s] = p.bs[bs_base + kbc * p.bs_ks];
+            }
+        }
+    };
+    auto take_scales = [&]() {
+        if constexpr (C::BLOCK_SCALE) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+#pragma unroll
+                for (int j = 0; j < NLD; ++j) as_cur[s][j] = as_nxt[s][j];
+                bs_cur[s] = bs_nxt[s];
+            }
+        }
+    };
+    auto compute = [&](int s) {
+        if constexpr (C::BLOCK_SCALE) {
+            float f[C::TM];
 #pragma unroll
             for (int a = 0; a < C::TM; ++a)
-                acc[a][b] = mma128<C::ARITH>(fb[s][b][0], fb[s][b][1], fa[s][a][0], fa[s][a][1], acc[a][b]);
+                f[a] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((((16 * a) & 63) + (lane & 15)) * 4,
+                                                                                as_cur[s][(16 * a) / 64])) * bs_cur[s];
+#pragma unroll
+            for (int b = 0; b < C::TN; ++b)
+#pragma unroll
+                for (int a = 0; a < C::TM; ++a) {
+                    const v4f part = mma128<C::ARITH>(fb[s][b][0], fb[s][b][1], fa[s][a][0], fa[s][a][1], v4f{0, 0, 0, 0});
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[a][b][r] += part[r] * f[a];
+                }
+        } else {
+#pragma unroll
+            for (int b = 0; b < C::TN; ++b)
+#pragma unroll
+                for (int a = 0; a < C::TM; ++a)
+                    acc[a][b] = mma128<C::ARITH>(fb[s][b][0], fb[s][b][1], fa[s][a][0], fa[s][a][1], acc[a][b]);
+        }
     };
 
     // ---- one round = steps k and k + 8 of this wave.  Ring programs by tile height (slots per step: A 2 TM, B 4):
@@ -142,6 +203,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     // the trip to HBM, and its slots turn over while B is still on its way.
     constexpr int SA = C::SA, SB = C::SB;
     auto start_round = [&](int k) {
+        fetch_scales(k);
+        __builtin_amdgcn_sched_barrier(0);          // (the scale loads stay in front of the copies)
         if constexpr (C::TM <= 2) {
             copy_b(k, 0);
             copy_b(k + C::NW, SB);
@@ -161,6 +224,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     // everything of the round into registers, the MFMAs of its first step, and (next: the round after this one
     // exists) the first copies of the next round as soon as the ring is empty; the MFMAs of the second step last
     auto finish_round = [&](int k, bool next, bool two) {
+        take_scales();
         if constexpr (C::TM <= 2) {
             wait_landed<SA>();
             drain_b(0, 0);

@@ -309,7 +309,7 @@ int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps
 int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
                    bool may_split, uint32_t *nsplit_out) {
     const int vi = choose_tile(tab, count, M, N, ksteps, block, kmaj, cus, may_split, nsplit_out);
-    if (vi < 0 || block || kmaj || M > 128 || tab[vi].bn != 32 || tab[vi].kgroups != 1) return vi;
+    if (vi < 0 || kmaj || M > 128 || tab[vi].bn != 32 || tab[vi].kgroups != 1) return vi;
     if (ksteps < 8 || (ksteps < 16 && M > 16)) return vi;
     for (int i = 0; i < count; ++i)
         if (tab[i].kgroups == 8 && (size_t)tab[i].bm >= M) {        // (rows of the table in ascending height)

@@ -108,11 +108,11 @@ def test_plan_names_the_kernel_without_a_device():
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
         assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
     assert plan(Q.DT_BF16, 0, 0, 24, 4096, 4096) == "skinny_32x32_k8"
-    # ... but not with few K steps, with block scales, or where the estimate prefers wide tiles
+    # ... but not with few K steps or where the estimate prefers wide tiles
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 7168, 512) == "128x32_w4x1_dma"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 8192, 1024) == "64x32_w4x1_dma"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 1024, 1024) == "skinny_16x32_k8"
-    assert "skinny" not in plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 64, 7168, 2048)
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 64, 7168, 2048) == "skinny_64x32_k8"          # block scales too
     assert "skinny" not in plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 28672, 4096)
     # mid sizes: the cost estimate prefers 128 x 128 tiles while they fit in one round of two per CU, and the
     # form with two K groups per workgroup where there are no more tiles than CUs
@@ -129,7 +129,7 @@ def test_plan_names_the_kernel_without_a_device():
     # ... also when a single launch would take smaller tiles for everything, and with a rest of at most 128 rows
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 5000, 4096, 7168) == "256x256_w2x2_solo+128x128_w2x2_k2"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 7000, 7168, 2048) == "256x256_w2x2_solo+skinny_128x32_k8"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 7000, 7168, 2048) == "256x256_w2x4_solo8_ks+128x32_w4x1_dma"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 7000, 7168, 2048) == "256x256_w2x4_solo8_ks+skinny_128x32_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 4096, 14336, 4096) == "256x256_w2x2_solo"     # 3.5 rounds: no gain
     Q.set_option("row_split", 0)
     try:

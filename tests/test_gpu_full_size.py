@@ -155,6 +155,53 @@ def test_cfg5_skinny_split_k(M):
     assert_close(host(cb), fref, what=Q.last_config())
 
 
+@pytest.mark.parametrize("shape", [(16, 7168, 2048), (96, 7168, 2048), (128, 7168, 2048 + 128), (37, 2080, 2048)])
+def test_block_scaled_skinny_m(shape):
+    """The skinny-M kernel with 128-block scales (the arithmetic of FP8_GEMM_kernel, hip_mix_gemm_kernel.cpp:231-244,
+    at decode-sized M): the whole matrix against the oracle with a_scale K-contiguous (QGEMM_LAYOUT_K_CONTIGUOUS) and,
+    in the reference's storage (QGEMM_LAYOUT_REFERENCE), rows-contiguous: the kernel reads it through strides, so the two give the same
+    bits.  K steps that do not divide by the 16 of a round, a ragged last strip and a last b_scale block that is not
+    whole; and power-of-two scales on small integers, where every product and sum is exact, bit for bit."""
+    M, N, K = shape
+    say("block-scaled skinny", shape)
+    KB, NB = K // 128, (N + 127) // 128
+    qa, _ = R.quantize_fp8(R.fill_normal((M, K), 61))
+    qb, _ = R.quantize_fp8(R.fill_normal((N, K), 62))
+    as_ = R.fill_uniform((M, KB), 63, 0.5, 2.0) / np.float32(448)
+    bs = R.fill_uniform((NB, KB), 64, 0.5, 2.0) / np.float32(448)
+    assert Q.plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, M, N, K).startswith("skinny")
+    ref = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)
+    c = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
+    name = Q.last_config()
+    assert name.startswith("skinny"), name
+    assert_close(host(c), ref, what=name)
+    # the reference's storage: operands and scales transposed; the NT kernel behind the operand transposes reads
+    # a_scale rows-contiguous
+    if M % 32 == 0 and N % 32 == 0:       # (the reference's dispatch refuses other shapes in its own layout: mix_gemm.h)
+        Q.set_option("kmajor", 0)
+        try:
+            c2 = torch.full((M, N), 9.0, dtype=torch.bfloat16, device="cuda")
+            Q.scaled_gemm(fp8_tensor(np.ascontiguousarray(qa.T)), fp8_tensor(np.ascontiguousarray(qb.T)),
+                          dev(np.ascontiguousarray(as_.T)), dev(np.ascontiguousarray(bs.T)), c2, M, N, K, Q.SCALE_BLOCK128,
+                          layout=Q.LAYOUT_REFERENCE)
+            assert "skinny" in Q.last_config(), Q.last_config()
+            assert torch.equal(c, c2), Q.last_config()
+        finally:
+            Q.set_option("kmajor", 1)
+    # power-of-two scales, small integers: exact in any order of summation
+    rng = np.random.default_rng(65)
+    ia = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    ib = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    as2 = np.exp2(rng.integers(-3, 4, (M, KB))).astype(np.float32)
+    bs2 = np.exp2(rng.integers(-3, 4, (NB, KB))).astype(np.float32)
+    ref2 = R.gemm_fp8_block(ia, ib, as2, bs2)
+    cx = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.scaled_gemm(fp8_tensor(R.encode_fp8(ia)), fp8_tensor(R.encode_fp8(ib)), dev(as2), dev(bs2), cx, M, N, K, Q.SCALE_BLOCK128)
+    assert Q.last_config().startswith("skinny"), Q.last_config()
+    assert np.array_equal(host(cx), ref2)
+
+
 def test_row_split_of_a_partly_empty_last_round():
     """4608 x 7680 are 540 tiles of 256 x 256 on 256 CUs: the rows of the two full rounds (4352) go to the 256 x 256
     kernel, the 256 rows below to a second launch with smaller tiles.  int8: the same integers as the single
