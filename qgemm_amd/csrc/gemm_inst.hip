@@ -100,17 +100,17 @@ static const Variant kTable[] = {
     ROW("16x32_w1x2_dma", 16, 32, 1, 2, LOAD_DMA, true),
     // 128 x 128 with eight waves in two K groups (GemmCfg::KG) and four stages (128 KiB: one workgroup per CU): for
     // shapes with no more tiles than CUs, where the two-stage row above would sit alone on its CU
-#if INST_BLOCK || INST_KMAJ      // (no block-scale or K-major form: alias, so indices agree across families)
+#if INST_KMAJ      // (no K-major form: alias, so indices agree across families)
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #else
-    row_of<true, GemmCfg<INST_ARITH, false, 128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 4, 2>,
+    row_of<true, GemmCfg<INST_ARITH, (bool)INST_BLOCK, 128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 4, 2>,
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("128x128_w2x2_k2", true),
 #endif
     // the same for the 64 x 128 tile, with six stages (two turns of copies in flight)
-#if INST_BLOCK || INST_KMAJ
+#if INST_KMAJ
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #else
-    row_of<true, GemmCfg<INST_ARITH, false, 64, 128, 1, 4, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 6, 2>,
+    row_of<true, GemmCfg<INST_ARITH, (bool)INST_BLOCK, 64, 128, 1, 4, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 6, 2>,
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("64x128_w1x4_k2", true),
 #endif
     // skinny M (gemm_skinny.cuh): the K split inside the workgroup, no staging, no barrier in the K loop

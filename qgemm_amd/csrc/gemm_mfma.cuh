@@ -152,12 +152,16 @@ struct GemmCfg {
                                   : (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE || BM * BN > 64 * 128 || KMAJ_ != 0) ? 2
                                   : (NSTAGE_FIT < NSTAGE_CNT ? (NSTAGE_FIT < 8 ? NSTAGE_FIT : 8)
                                                              : (NSTAGE_CNT < 8 ? NSTAGE_CNT : 8));
-    static constexpr int LDS_BYTES = A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES;
-    static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && !BLOCK_SCALE && KMAJ_ == 0 && STAGES_ >= 2 &&
-                                   STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
+    // Block scales with K groups: the a_scale values of a stage (one float per tile row, at most 128) travel to LDS
+    // like the operands, 512 bytes per stage behind the ring, so that every copy of the loop is of one kind and the
+    // wave's own count of copies in flight stays exact (a register load among them makes the compiler wait for all).
+    static constexpr int SCALE_LDS = (BLOCK_SCALE_ && KGROUPS_ == 2) ? NSTAGE * 512 : 0;
+    static constexpr int LDS_BYTES = (A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES) + SCALE_LDS;
+    static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && (!BLOCK_SCALE || KGROUPS_ == 2) && KMAJ_ == 0 &&
+                                   STAGES_ >= 2 && STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
                   "explicit stage count: simple pipeline, DMA loader, within LDS and the 6-bit counter");
-    static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && !BLOCK_SCALE && KMAJ_ == 0 &&
-                                    NSTAGE >= 4 && NSTAGE % 2 == 0),
+    static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && KMAJ_ == 0 &&
+                                    NSTAGE >= 4 && NSTAGE % 2 == 0 && (!BLOCK_SCALE_ || (BM_ <= 128 && BN_ <= 128))),
                   "K groups: simple pipeline, DMA loader, an even number (at least four) of stages");
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
     static_assert(NLOAD % NW == 0, "load instructions must divide evenly over the waves");
@@ -1000,6 +1004,16 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     } else {
         constexpr int NS = C::NSTAGE;
+        // The barrier of a step.  With the DMA loader it is the bare s_barrier behind the wave's own wait for its
+        // copies (counted, see below): __syncthreads() carries a fence that the compiler turns into "wait for every
+        // copy in flight", which empties the ring at every step and leaves the stages issued ahead no time to land
+        // under the MFMAs.  Fragment reads are complete before their MFMAs issue, so a wave that reaches the barrier
+        // has left the buffers the next copies overwrite.  (Register staging writes LDS with ds_write and needs the
+        // full barrier; so do the K-major tiles, whose transposing reads the compiler orders behind all copies.)
+        auto ring_barrier = [&]() {
+            if constexpr (C::LOADER == LOAD_DMA && C::KMAJ == 0) phase_barrier();
+            else __syncthreads();
+        };
         // Small tiles with a deep ring (NS >= 4): two K steps per barrier.  A workgroup of these is alone or nearly
         // alone on its CU and every step is a chain wait -> barrier -> fragment reads -> a handful of MFMAs, about
         // 0.25 - 0.36 us; taking the steps in pairs pays the barrier and the LDS latency once for two.  Before turn
@@ -1012,17 +1026,38 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // stages in flight are 64 KiB per CU: at the latency of a copy that misses the L2 that bounds a turn
             // from below.  Touching the lines of later turns with plain loads, so that the copies would find them
             // in the L2, was tried and made the loop a quarter slower.)
+            // Block scales: every wave adds one 4-byte-per-lane copy per stage that brings the a_scale values of 64 tile
+            // rows (even waves rows 0 - 63, odd waves rows 64 - 127: the same bytes to the same place from several
+            // waves, so that all waves count alike) to the stage's 512 bytes behind the ring.
+            constexpr int CPS = C::LPT + (C::BLOCK_SCALE ? 1 : 0);          // copies per stage and wave
+            const uint32_t as_voff_k2 = (row0 + 64 * (wave & 1) + lane) * p.as_ms * 4;
+            auto issue_stage_k2 = [&](int kt) {
+                issue_stage(kt);
+                if constexpr (C::BLOCK_SCALE) {
+                    lds_void *dst = (lds_void *)(smem + NS * C::STAGE_BYTES + (kt % NS) * 512 + (wave & 1) * 256);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 4, as_voff_k2, (kbeg + (uint32_t)kt) * p.as_ks * 4, 0, 0);
+                }
+            };
 #pragma unroll
             for (int j = 0; j < NS - 2; ++j)
-                if (j < nk) issue_stage(j);
+                if (j < nk) issue_stage_k2(j);
             for (int kt = 0; kt < nk; kt += 2) {
-                if (kt + NS - 2 <= nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 4) * C::LPT));
+                if (kt + NS - 2 <= nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 4) * CPS));
                 else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-                __syncthreads();
-                if (kt + NS - 2 < nk) issue_stage(kt + NS - 2);
-                if (kt + NS - 1 < nk) issue_stage(kt + NS - 1);
+                ring_barrier();
                 const int mine = kt + kg;
+                if (kt + NS - 2 < nk) issue_stage_k2(kt + NS - 2);
+                if (kt + NS - 1 < nk) issue_stage_k2(kt + NS - 1);
                 if (mine < nk) {
+                    if constexpr (C::BLOCK_SCALE) {
+                        const char *sc = smem + NS * C::STAGE_BYTES + (mine % NS) * 512 + (wm * C::WM + (lane & 15)) * 4;
+#pragma unroll
+                        for (int a = 0; a < C::TM; ++a) as_cur[a] = *(const float *)(sc + a * 64);
+                        const uint32_t kb = kbeg + (uint32_t)mine;
+#pragma unroll
+                        for (int j = 0; j < NBS; ++j)
+                            bs_cur[j] = p.bs[__builtin_amdgcn_readfirstlane(bs_off[j] + kb * p.bs_ks)];
+                    }
                     const char *st = smem + (mine % NS) * C::STAGE_BYTES;
                     v4i fa[C::TM][2], fb[C::TN][2];
 #pragma unroll
@@ -1038,8 +1073,18 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #pragma unroll
                     for (int b = 0; b < C::TN; ++b)
 #pragma unroll
-                        for (int a = 0; a < C::TM; ++a)
-                            acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                        for (int a = 0; a < C::TM; ++a) {
+                            if constexpr (C::BLOCK_SCALE) {
+                                // P * (as * bs), then accumulate (hip_mix_gemm_kernel.cpp:241 has (P * as) * bs: the
+                                // factor formed first is one multiply per row and K block instead of four per MFMA)
+                                const v4f part = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                                const float f = as_cur[a] * bs_cur[(b * 16) / 128];
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) acc[a][b][r] += part[r] * f;
+                            } else {
+                                acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                            }
+                        }
                 }
             }
         } else if constexpr (PAIRS) {
@@ -1049,7 +1094,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             for (int kt = 0; kt < nk; kt += 2) {
                 if (kt + NS - 2 <= nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 4) * C::LPT));
                 else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
-                __syncthreads();
+                ring_barrier();
                 if (kt + NS - 2 < nk) issue_stage(kt + NS - 2);
                 if (kt + NS - 1 < nk) issue_stage(kt + NS - 1);
                 const bool two = kt + 1 < nk;
@@ -1109,7 +1154,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 if (NS > 2 && kt + NS - 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * C::LPT));
                 else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
             }
-            __syncthreads();                                 // ... and everybody else's; tile kt-1 is fully consumed
+            ring_barrier();                                  // ... and everybody else's; tile kt-1 is fully consumed
             expand_scales();
             auto next_stage = [&]() {                        // into the buffer tile kt-1 has just left
                 if (kt + NS - 1 < nk) {
@@ -1150,11 +1195,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #pragma unroll
                 for (int a = 0; a < C::TM; ++a) {
                     if constexpr (C::BLOCK_SCALE) {
-                        // (P * as) * bs, then accumulate: hip_mix_gemm_kernel.cpp:241
+                        // P * (as * bs), then accumulate (hip_mix_gemm_kernel.cpp:241 has (P * as) * bs: the factor
+                        // formed first is one multiply per row and K block instead of four per MFMA)
                         const v4f part = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                        const float sa = as_cur[a], sb = bs_cur[(b * 16) / 128];
+                        const float f = as_cur[a] * bs_cur[(b * 16) / 128];
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[a][b][r] += (part[r] * sa) * sb;
+                        for (int r = 0; r < 4; ++r) acc[a][b][r] += part[r] * f;
                     } else {
                         acc[a][b] = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], acc[a][b]);
                     }

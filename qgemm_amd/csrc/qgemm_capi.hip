@@ -244,7 +244,7 @@ bool mfma_shape_ok(const NtProblem &q) {
 // (K steps x time per step + a fixed prologue / epilogue), a last partial round that leaves a 128 x 128
 // workgroup alone on its CU runs its steps faster, and a K split pays a second launch plus the traffic of the
 // partial planes.  The times per 128-byte K step were read off a sweep of every variant over square and oblong
-// shapes from 1024 to 8192 (fp8 and bf16 agree per step; block scales cost about a third more): 1.25 us for the
+// shapes from 1024 to 8192 (fp8 and bf16 agree per step; block scales have figures of their own): 1.25 us for the
 // 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.52 us for the 128 x 128
 // row with two K groups (one per CU: it only wins where there are no more tiles than CUs), 0.52 us for 64 x 128 and
 // 0.40 us for its row with two K groups (graph replays of 384 / 512 x 4096 x 4096 and 1024 x 2048 x 7168), 0.39 us for
@@ -258,10 +258,17 @@ struct TileModel {
     int bm, bn, per_cu;
     double step_shared, step_alone, fixed;     // microseconds
     bool kgroups;                              // the row of this tile with two K groups per workgroup (GemmCfg::KG)
+    // the same with 128-block scales (fp8): the fold costs the 8-wave 256 x 256 kernel a tenth, the simple pipeline
+    // more (its block-scaled rows have two stages, so more workgroups share a CU), the K-group rows most
+    int blk_per_cu;
+    double blk_shared, blk_alone;
 };
-const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false}, {128, 128, 2, 0.85, 0.66, 2.0, false},
-                                 {128, 128, 1, 0.52, 0.52, 3.0, true},  {64, 128, 1, 0.52, 0.52, 1.5, false},
-                                 {64, 128, 1, 0.40, 0.40, 2.5, true},   {128, 32, 1, 0.39, 0.39, 1.0, false}};
+// (block scales, graph replays: 256 x 256 2048 x 4608 x 7168 77 us, 1536 x 7168 x 2048 27.6; 128 x 128 1024 x 7168 x 2048 25.9,
+// 1024 x 4608 x 7168 75.0; 64 x 128 1024 x 4608 x 7168 69.9, 512 x 4608 x 7168 47.8; K groups 512 x 7168 x 2048 16.8 and 12.9 for
+// 256 rows; 128 x 32 256 x 7168 x 2048 12.9)
+const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.40, 1.10},
+                                 {128, 128, 1, 0.52, 0.52, 3.0, true, 1, 0.92, 0.92},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
+                                 {64, 128, 1, 0.40, 0.40, 2.5, true, 1, 0.72, 0.72},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
 // rows with two K groups: eight waves on a tile that otherwise has four (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 
@@ -277,11 +284,11 @@ int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t kst
         const size_t tiles = ((M + tm.bm - 1) / tm.bm) * ((N + tm.bn - 1) / tm.bn);
         for (uint32_t ns = 1; ns <= 8; ns *= 2) {
             if (ns > 1 && (!may_split || ksteps / ns < 4)) break;
-            const size_t wgs = tiles * ns, slots = (size_t)cus * tm.per_cu, steps = (ksteps + ns - 1) / ns;
+            const size_t wgs = tiles * ns, slots = (size_t)cus * (block ? tm.blk_per_cu : tm.per_cu), steps = (ksteps + ns - 1) / ns;
             const size_t full = wgs / slots, rem = wgs % slots;
-            const double scale = block ? 1.35 : 1.0;
-            double t = (double)full * (steps * tm.step_shared * scale + tm.fixed);
-            if (rem) t += steps * (rem <= (size_t)cus ? tm.step_alone : tm.step_shared) * scale + tm.fixed;
+            const double shared = block ? tm.blk_shared : tm.step_shared, alone = block ? tm.blk_alone : tm.step_alone;
+            double t = (double)full * (steps * shared + tm.fixed);
+            if (rem) t += steps * (rem <= (size_t)cus ? alone : shared) + tm.fixed;
             if (ns > 1) t += 4.0 + (double)M * N * 4.0 * (ns + 1) / 3.0e6;
             if (best < 0 || t < best_t) {
                 best = vi;
