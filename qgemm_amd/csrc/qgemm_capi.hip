@@ -247,7 +247,7 @@ bool mfma_shape_ok(const NtProblem &q) {
 // shapes from 1024 to 8192 (fp8 and bf16 agree per step; block scales have figures of their own): 1.25 us for the
 // 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.52 us for the 128 x 128
 // row with two K groups (one per CU: it only wins where there are no more tiles than CUs), 0.52 us for 64 x 128 and
-// 0.40 us for its row with two K groups (graph replays of 384 / 512 x 4096 x 4096 and 1024 x 2048 x 7168), 0.39 us for
+// 0.36 us for its row with two K groups (graph replays of 384 / 512 x 4096 x 4096 and 1024 x 2048 x 7168), 0.39 us for
 // 128 x 32.  A K split adds 4 us and the partial planes at 3 TB/s.
 //
 // M <= 64 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
@@ -268,7 +268,7 @@ struct TileModel {
 // 256 rows; 128 x 32 256 x 7168 x 2048 12.9)
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.40, 1.10},
                                  {128, 128, 1, 0.52, 0.52, 3.0, true, 1, 0.92, 0.92},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
-                                 {64, 128, 1, 0.40, 0.40, 2.5, true, 1, 0.72, 0.72},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
+                                 {64, 128, 1, 0.36, 0.36, 2.5, true, 1, 0.72, 0.72},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
 // rows with two K groups: eight waves on a tile that otherwise has four (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 
