@@ -103,7 +103,7 @@ static const Variant kTable[] = {
 #if INST_KMAJ      // (no K-major form: alias, so indices agree across families)
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #else
-    row_of<true, GemmCfg<INST_ARITH, (bool)INST_BLOCK, 128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 4, 2>,
+    row_of<true, GemmCfg<INST_ARITH, (bool)INST_BLOCK, 128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, INST_BLOCK ? 4 : 5, 2>,
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("128x128_w2x2_k2", true),
 #endif
     // the same for the 64 x 128 tile, with six stages (two turns of copies in flight)

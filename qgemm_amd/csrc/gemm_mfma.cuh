@@ -161,8 +161,8 @@ struct GemmCfg {
                                    STAGES_ >= 2 && STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
                   "explicit stage count: simple pipeline, DMA loader, within LDS and the 6-bit counter");
     static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && KMAJ_ == 0 &&
-                                    NSTAGE >= 4 && NSTAGE % 2 == 0 && (!BLOCK_SCALE_ || (BM_ <= 128 && BN_ <= 128))),
-                  "K groups: simple pipeline, DMA loader, an even number (at least four) of stages");
+                                    NSTAGE >= 4 && (!BLOCK_SCALE_ || (BM_ <= 128 && BN_ <= 128))),
+                  "K groups: simple pipeline, DMA loader, at least four stages");
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
     static_assert(NLOAD % NW == 0, "load instructions must divide evenly over the waves");
     static_assert(!BLOCK_SCALE || ARITH == AR_F8, "block scales are defined for fp8 only");
