@@ -98,8 +98,9 @@ static const Variant kTable[] = {
     ROW("128x32_w4x1_dma", 128, 32, 4, 1, LOAD_DMA, true),
     ROW("64x32_w4x1_dma", 64, 32, 4, 1, LOAD_DMA, true),
     ROW("16x32_w1x2_dma", 16, 32, 1, 2, LOAD_DMA, true),
-    // 128 x 128 with eight waves in two K groups (GemmCfg::KG) and four stages (128 KiB: one workgroup per CU): for
-    // shapes with no more tiles than CUs, where the two-stage row above would sit alone on its CU
+    // 128 x 128 with eight waves in two K groups (GemmCfg::KG) and five stages (160 KiB, one workgroup per CU; four
+    // with block scales, whose a_scale values take 2 KiB behind the ring): for shapes with no more tiles than CUs,
+    // where the two-stage row above would sit alone on its CU
 #if INST_KMAJ      // (no K-major form: alias, so indices agree across families)
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #else
@@ -127,7 +128,7 @@ static const Variant kTable[] = {
 #endif
     // the block-scaled 8-wave solo kernel reading a_scale with the K blocks contiguous, as QGEMM_LAYOUT_K_CONTIGUOUS
     // passes it (GemmCfg::ASK): launch_nt swaps it in for the row above of the same name when the scales allow it,
-    // which saves the transposed copy of a_scale that the other kernels need
+    // which saves a transposed copy of a_scale (the simple and ping-pong pipelines read it through strides)
 #if INST_BLOCK && !INST_KMAJ
     row_of<true, GemmCfg<INST_ARITH, true, 256, 256, 2, 4, LOAD_DMA, PIPE_SOLO, 0, true, 0, 0, 1, true>,
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("256x256_w2x4_solo8_ks", false),

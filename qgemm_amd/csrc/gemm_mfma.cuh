@@ -144,7 +144,8 @@ struct GemmCfg {
     static constexpr int LPT_A = RBA * 2 / NW;                  // A load instructions per wave (ping-pong)
     // simple pipeline with the DMA loader: as many stages in flight as LDS and the 6-bit vmcnt allow (at most
     // 8).  A workgroup that streams a narrow strip of B (skinny M) otherwise waits one full memory round trip
-    // per K step.  The block-scale form keeps two (its scale loads share vmcnt with the copies).
+    // per K step.  The block-scale form keeps two (its scale loads share vmcnt with the copies), except with K
+    // groups, where the scales travel to LDS like the operands.
     static constexpr int NSTAGE_FIT = (160 * 1024) / STAGE_BYTES, NSTAGE_CNT = 2 + 63 / LPT;
     // Only for the small tiles: a 128 x 128 tile with two stages leaves room for two workgroups per CU, which is
     // worth more to a compute-bound shape than deeper prefetch.

@@ -311,7 +311,8 @@ int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps
 // against skinny kernel: 16 x 7168 x 2048 7.6 / 5.4, 64 x 7168 x 2048 9.0 / 6.7, 128 x 7168 x 2048 11.0 / 8.2,
 // 16 x 7168 x 8192 24.6 / 15.2, 32 x 4096 x 4096 12.7 / 8.3, 128 x 4096 x 4096 18.3 / 12.5, 16 x 1024 x 1024
 // 5.6 / 3.1; with K = 1024 and more than 16 rows or K = 512 the narrow tiles stay ahead (64 x 8192 x 1024 5.0 / 5.2,
-// 128 x 7168 x 512 4.6 / 6.0).  It never wants a K split on top: one makes it slower wherever it was tried.
+// 128 x 7168 x 512 4.6 / 6.0).  It never wants a K split on top: one makes it slower wherever it was tried.  The same
+// rule serves block scales (B resident: 16 x 7168 x 2048 10.8 / 6.6, 128 x 7168 x 2048 15.7 / 9.5).
 // kmaj: the table is a K-major family, which has no narrow tiles: the estimate then serves every M
 int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
                    bool may_split, uint32_t *nsplit_out) {
