@@ -26,7 +26,7 @@
 
 namespace qgemm {
 
-template <int ARITH_, int TM_, bool BLOCK_SCALE_ = false>
+template <int ARITH_, int TM_, bool BLOCK_SCALE_ = false, int TN_ = 2>
 struct SkinnyCfg {
     static constexpr int ARITH = ARITH_;
     // 128-block scales (fp8): every MFMA starts from zero and its product of one K block is folded into the running
@@ -36,14 +36,17 @@ struct SkinnyCfg {
     // copies, so they have arrived wherever the copies they precede have.
     static constexpr bool BLOCK_SCALE = BLOCK_SCALE_;
     static_assert(!BLOCK_SCALE_ || ARITH_ == AR_F8, "block scales are defined for fp8 only");
-    static constexpr int TM = TM_, TN = 2;                  // 16 x 16 MFMA tiles of the workgroup's tile
-    static constexpr int BM = 16 * TM_, BN = 32;
+    // TN = 4 (with TM = 4: a 64 x 64 tile): half the strips, so A is fetched half as often; for shapes with several
+    // row tiles, where a CU's load path, not the stream of B from HBM, is what bounds a 32-column strip.
+    static constexpr int TM = TM_, TN = TN_;                // 16 x 16 MFMA tiles of the workgroup's tile
+    static constexpr int BM = 16 * TM_, BN = 16 * TN_;
     static constexpr int NW = 8, THREADS = NW * kWave;
     static constexpr int SLOTS = 20;                        // ring slots (1 KiB = one copy instruction) per wave
     static constexpr int SA = 2 * TM, SB = 2 * TN;          // slots of one step of A / of B
     static constexpr int RING_BYTES = SLOTS * 1024;
     static constexpr int LDS_BYTES = NW * RING_BYTES;       // the rings; afterwards one partial sum (1 KiB per tile) per wave
     static_assert(TM == 1 || TM == 2 || TM == 4 || TM == 8, "the programs below are written for these tile heights");
+    static_assert(TN == 2 || (TN == 4 && TM == 4 && !BLOCK_SCALE_), "64-column strips: the 64 x 64 tile, per-matrix scales");
     static_assert(TM * TN * 1024 <= RING_BYTES, "a wave's partial sums fit its ring");
 };
 
@@ -71,7 +74,17 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
         wg = __builtin_amdgcn_readfirstlane(wg / p.nsplit);
     }
     // column strips side by side (the few row tiles of one strip are neighbours: they share the strip of B in L2)
-    const uint32_t tm = __builtin_amdgcn_readfirstlane(wg % p.tiles_m), tn = __builtin_amdgcn_readfirstlane(wg / p.tiles_m);
+    // (the 64 x 64 form has many row tiles: there the tiles an XCD holds at one time form a compact block, as in
+    // gemm_nt_kernel, so that its L2 fetches each panel of A and B once)
+    uint32_t tm, tn;
+    if constexpr (C::TN == 4) {
+        tile_map(wg, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+        tm = __builtin_amdgcn_readfirstlane(tm);
+        tn = __builtin_amdgcn_readfirstlane(tn);
+    } else {
+        tm = __builtin_amdgcn_readfirstlane(wg % p.tiles_m);
+        tn = __builtin_amdgcn_readfirstlane(wg / p.tiles_m);
+    }
     const uint32_t row0 = tm * C::BM, col0 = tn * C::BN;
     const uint32_t kbeg = z * p.ksteps_per_split;
     const uint32_t kend = kbeg + p.ksteps_per_split < p.ksteps ? kbeg + p.ksteps_per_split : p.ksteps;
@@ -99,12 +112,13 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void *)(ring + (slot + i) * 1024), 16, voff_a,
                                                      (first + i) * 8 * p.lda + (uint32_t)kt * 128, 0, 0);
     };
-    auto copy_b = [&](int kt, int slot) {
+    auto copy_b_part = [&](int kt, int first, int n, int slot) {
 #pragma unroll
-        for (int i = 0; i < C::SB; ++i)
+        for (int i = 0; i < n; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void *)(ring + (slot + i) * 1024), 16, voff_b,
-                                                     i * 8 * p.ldb + (uint32_t)kt * 128, 0, 0);
+                                                     (first + i) * 8 * p.ldb + (uint32_t)kt * 128, 0, 0);
     };
+    auto copy_b = [&](int kt, int slot) { copy_b_part(kt, 0, C::SB, slot); };
     // fragments of the two steps of a round: [step][block][half]
     v4i fa[2][C::TM][2], fb[2][C::TN][2];
     auto drain_a = [&](int s, int blk0, int nblk, int slot) {       // blocks blk0 .. of step s sit in ring slots slot ..
@@ -114,13 +128,14 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
             fa[s][blk0 + i][1] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off1);
         }
     };
-    auto drain_b = [&](int s, int slot) {
+    auto drain_b_part = [&](int s, int blk0, int nblk, int slot) {
 #pragma unroll
-        for (int i = 0; i < C::TN; ++i) {
-            fb[s][i][0] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off0);
-            fb[s][i][1] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off1);
+        for (int i = 0; i < nblk; ++i) {
+            fb[s][blk0 + i][0] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off0);
+            fb[s][blk0 + i][1] = *(const v4i *)(ring + slot * 1024 + i * 2048 + off1);
         }
     };
+    auto drain_b = [&](int s, int slot) { drain_b_part(s, 0, C::TN, slot); };
     auto drained = [&]() {                                  // the fragment reads are done: their slots may be refilled
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());
@@ -199,13 +214,19 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     //   TM == 4  (24 slots):  A0 B0 B1 A1[0..4)  | A0 drained ->  A1[4..8)
     //   TM == 8  (40 slots):  A0[0..12) B0 B1    | A0[0..12) drained -> A0[12..16) A1[0..8) | B0 B1 A0[12..16) drained
     //                         -> A1[8..16)
+    //   TM == 4, TN == 4 (32 slots, B 8 per step):  A0 B0 B1[0..4) | A0 drained -> B1[4..8) A1[0..4) | B0 drained
+    //                         -> A1[4..8)
     // A goes in front of B where the ring cannot take the round at once: the wait for it then does not include
     // the trip to HBM, and its slots turn over while B is still on its way.
     constexpr int SA = C::SA, SB = C::SB;
     auto start_round = [&](int k) {
         fetch_scales(k);
         __builtin_amdgcn_sched_barrier(0);          // (the scale loads stay in front of the copies)
-        if constexpr (C::TM <= 2) {
+        if constexpr (C::TN == 4) {                   // 64 x 64: A0 B0 B1[0..4) fill the ring
+            copy_a(k, 0, 8, 0);
+            copy_b(k, 8);
+            copy_b_part(k + C::NW, 0, 4, 16);
+        } else if constexpr (C::TM <= 2) {
             copy_b(k, 0);
             copy_b(k + C::NW, SB);
             copy_a(k, 0, SA, 2 * SB);
@@ -225,7 +246,27 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     // exists) the first copies of the next round as soon as the ring is empty; the MFMAs of the second step last
     auto finish_round = [&](int k, bool next, bool two) {
         take_scales();
-        if constexpr (C::TM <= 2) {
+        if constexpr (C::TN == 4) {
+            // ring: A0 0-7, B0 8-15, B1a 16-19 | A0 drained -> B1b 0-3, A1a 4-7 | B0 drained -> A1b 8-11
+            wait_landed<12>();
+            drain_a(0, 0, 4, 0);
+            drained();
+            copy_b_part(k + C::NW, 4, 4, 0);
+            copy_a(k + C::NW, 0, 4, 4);
+            wait_landed<12>();
+            drain_b(0, 8);
+            drained();
+            copy_a(k + C::NW, 4, 4, 8);
+            compute(0);
+            wait_landed<12>();
+            drain_b_part(1, 0, 2, 16);
+            wait_landed<8>();
+            drain_b_part(1, 2, 2, 0);
+            wait_landed<4>();
+            drain_a(1, 0, 2, 4);
+            wait_landed<0>();
+            drain_a(1, 2, 2, 8);
+        } else if constexpr (C::TM <= 2) {
             wait_landed<SA>();
             drain_b(0, 0);
             drain_b(1, SB);

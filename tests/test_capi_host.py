@@ -94,7 +94,8 @@ def test_plan_names_the_kernel_without_a_device():
     """qgemm_plan: the tile / pipeline / K-split choice for the five BASELINE configs and for operands stored
     K-major, from the host (256 CUs assumed).  Pins the heuristic: a change of choice shows up here first."""
     plan = Q.plan
-    assert plan(Q.DT_F16, 0, 0, 1024, 1024, 1024) == "128x32_w4x1_dma"                       # config 1
+    assert plan(Q.DT_F16, 0, 0, 1024, 1024, 1024) == "skinny_64x64_k8"                       # config 1
+    assert plan(Q.DT_F16, 0, 0, 1024, 1024, 512) == "128x32_w4x1_dma"                        # (8 K steps: one per wave)
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4096) == "256x256_w2x2_solo"     # config 2
     # int8 and 16-bit types: 4 waves when the tiles fill whole rounds of CUs, 8 waves in a partly filled round
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x4_solo8"
