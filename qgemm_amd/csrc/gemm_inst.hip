@@ -45,7 +45,7 @@ static hipError_t launch_skinny(const GemmArgs &a, uint32_t grid, hipStream_t s)
 // Picked by choose_variant in place of the narrow simple-pipeline tiles, never by the table scan (auto_ok = false).
 template <int TM, int TN = 2>
 static Variant skinny_row(const char *name) {
-    using C = SkinnyCfg<INST_ARITH, TM, (bool)INST_BLOCK && TN == 2, TN>;
+    using C = SkinnyCfg<INST_ARITH, TM, (bool)INST_BLOCK, TN>;
     return Variant{name, C::ARITH, C::BLOCK_SCALE, C::BM, C::BN, C::THREADS, C::LDS_BYTES, LOAD_DMA, false, 8, false,
                    C::BLOCK_SCALE, &launch_skinny<C>};
 }
@@ -136,7 +136,7 @@ static const Variant kTable[] = {
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #endif
     // the skinny-M kernel on a 64 x 64 tile: for shapes with a few row tiles whose 64 x 64 tiles fit one round of CUs
-#if INST_BLOCK || INST_KMAJ      // (per-matrix scales, K-contiguous operands only: alias, so indices agree across families)
+#if INST_KMAJ      // (K-contiguous operands only: alias, so indices agree across families)
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #else
     skinny_row<4, 4>("skinny_64x64_k8"),

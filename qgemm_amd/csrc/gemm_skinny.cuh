@@ -30,8 +30,8 @@ template <int ARITH_, int TM_, bool BLOCK_SCALE_ = false, int TN_ = 2>
 struct SkinnyCfg {
     static constexpr int ARITH = ARITH_;
     // 128-block scales (fp8): every MFMA starts from zero and its product of one K block is folded into the running
-    // sum with a_scale[row, kb] * b_scale[strip, kb], as in gemm_nt_kernel.  The strip of 32 columns lies inside one
-    // 128-column block of b_scale.  a_scale is read with the caller's strides (lane l: row l of the tile, the rows of
+    // sum with a_scale[row, kb] * b_scale[strip, kb], as in gemm_nt_kernel.  The strip of 32 (or 64) columns lies inside
+    // one 128-column block of b_scale.  a_scale is read with the caller's strides (lane l: row l of the tile, the rows of
     // an MFMA tile picked out of that with ds_bpermute); the scales of a round are requested in front of the round's
     // copies, so they have arrived wherever the copies they precede have.
     static constexpr bool BLOCK_SCALE = BLOCK_SCALE_;
@@ -46,7 +46,7 @@ struct SkinnyCfg {
     static constexpr int RING_BYTES = SLOTS * 1024;
     static constexpr int LDS_BYTES = NW * RING_BYTES;       // the rings; afterwards one partial sum (1 KiB per tile) per wave
     static_assert(TM == 1 || TM == 2 || TM == 4 || TM == 8, "the programs below are written for these tile heights");
-    static_assert(TN == 2 || (TN == 4 && TM == 4 && !BLOCK_SCALE_), "64-column strips: the 64 x 64 tile, per-matrix scales");
+    static_assert(TN == 2 || (TN == 4 && TM == 4), "64-column strips: the 64 x 64 tile");
     static_assert(TM * TN * 1024 <= RING_BYTES, "a wave's partial sums fit its ring");
 };
 

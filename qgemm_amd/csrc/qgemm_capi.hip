@@ -317,13 +317,14 @@ int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps
 int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
                    bool may_split, uint32_t *nsplit_out) {
     const int vi = choose_tile(tab, count, M, N, ksteps, block, kmaj, cus, may_split, nsplit_out);
-    // The same kernel on 64 x 64 tiles (per-matrix scales): shapes with several row tiles whose 64 x 64 tiles fit one
+    // The same kernel on 64 x 64 tiles: shapes with several row tiles whose 64 x 64 tiles fit one
     // round of CUs and give most of them work, 16 K steps or more.  Against whatever the estimate picks (narrow
     // tiles, K-group tiles with a K split) it is 13 - 33 % faster over 512 .. 2048 rows x 256 .. 3000 columns x 2 .. 8 KiB
     // of K (fp16 1024^3 7.3 -> 6.3 us, fp8 1000 x 1000 x 4096 13.1 -> 8.8), slower only with 8 K steps (one per wave)
     // or with 64 tiles and 64 K steps; beyond 64 K steps the tiles with a K split across workgroups catch up
-    // (bf16 256 x 2048 x 7168, 112 steps: 18.9 against 22.9 us).
-    if (vi >= 0 && !block && !kmaj && M > 128 && ksteps >= 16 && ksteps <= 64) {
+    // (bf16 256 x 2048 x 7168, 112 steps: 18.9 against 22.9 us).  With block scales the gain is larger, the small tiles
+    // of the simple pipeline being slower there: 512 x 2048 x 4096 18.3 -> 11.7 us, 256 x 4096 x 4096 17.8 -> 11.8.
+    if (vi >= 0 && !kmaj && M > 128 && ksteps >= 16 && ksteps <= 64) {
         const size_t t64 = ((M + 63) / 64) * ((N + 63) / 64);
         if (t64 <= (size_t)cus && (t64 >= 128 || (t64 >= 64 && ksteps <= 32)))
             for (int i = 0; i < count; ++i)

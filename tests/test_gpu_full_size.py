@@ -155,7 +155,8 @@ def test_cfg5_skinny_split_k(M):
     assert_close(host(cb), fref, what=Q.last_config())
 
 
-@pytest.mark.parametrize("shape", [(16, 7168, 2048), (96, 7168, 2048), (128, 7168, 2048 + 128), (37, 2080, 2048)])
+@pytest.mark.parametrize("shape", [(16, 7168, 2048), (96, 7168, 2048), (128, 7168, 2048 + 128), (37, 2080, 2048),
+                                   (512, 2048, 4096), (300, 1000, 2048 + 128)])        # (the last two: 64 x 64 tiles)
 def test_block_scaled_skinny_m(shape):
     """The skinny-M kernel with 128-block scales (the arithmetic of FP8_GEMM_kernel, hip_mix_gemm_kernel.cpp:231-244,
     at decode-sized M): the whole matrix against the oracle with a_scale K-contiguous (QGEMM_LAYOUT_K_CONTIGUOUS) and,
