@@ -25,6 +25,8 @@ def _draw(rng):
     fam = rng.choice(["i8", "f8", "f8_block", "f8_block_ref", "bf16_nk", "bf16_kn", "f16_nk", "f16_kn"])
     kq = {"i8": 128, "f8": 128, "f8_block": 128, "f8_block_ref": 128}.get(fam, 64)     # K bytes % 128 == 0
     K = int(rng.integers(1, 9)) * kq
+    if rng.random() < 0.25:                         # a long K: several rounds of the skinny-M kernel, deep rings
+        K = int(rng.integers(9, 41)) * kq
     if rng.random() < 0.3:
         M = int(rng.choice([1, 7, 16, 33, 100, 128]))
     else:
