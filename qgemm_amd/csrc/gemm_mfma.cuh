@@ -111,11 +111,11 @@ struct GemmCfg {
     // launch that would copy the scales into the other order.
     static constexpr bool AS_ANY_STRIDE = BLOCK_SCALE_ && PIPE_ != PIPE_SOLO;
     // STAGES (simple pipeline, DMA loader): number of LDS stages, 0 = chosen below.
-    // KGROUPS = 2: the workgroup has two sets of WAVES_M x WAVES_N waves; all of them copy, set 0 computes the
-    // even K steps and set 1 the odd ones of the same tile (one barrier per pair of steps), and the two partial
-    // sums meet in LDS before the epilogue.  A tile that is alone on its CU (a shape with no more tiles than CUs)
-    // otherwise reads its fragments and runs its MFMAs in turn, with nothing to overlap either with: two waves
-    // per SIMD working on different K steps do what a second workgroup on the CU would.
+    // KGROUPS = 2: the workgroup has two sets of WAVES_M x WAVES_N waves and two waves that copy; set 0 computes
+    // the even K steps and set 1 the odd ones of the same tile, half a turn apart, and the two partial sums meet in
+    // LDS before the epilogue.  A tile that is alone on its CU (a shape with no more tiles than CUs) otherwise
+    // reads its fragments and runs its MFMAs in turn, with nothing to overlap either with: two waves per SIMD
+    // working on different K steps do what a second workgroup on the CU would.
     static constexpr int KG = KGROUPS_;
     // KMAJ: which operands are stored K-major (bit 0: A is K x M with M contiguous, bit 1: B is K x N with N
     // contiguous) instead of K-contiguous.  A K-major tile keeps its rows of K in LDS and the MFMA fragments
@@ -133,7 +133,9 @@ struct GemmCfg {
     static constexpr int BM = BM_, BN = BN_, BKB = 128;         // BKB: bytes of K per step
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int NW = WAVES_M * WAVES_N * KGROUPS_;
-    static constexpr int THREADS = NW * kWave;
+    // K groups: four more waves that only copy (waves NW .. NW+3, see the K loop)
+    static constexpr int NPROD = KGROUPS_ == 2 ? 4 : 0;
+    static constexpr int THREADS = (NW + NPROD) * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
     static constexpr int TM = WM / 16, TN = WN / 16;            // 16x16 MFMA tiles per wave
     static constexpr int RBA = BM / 16, RBB = BN / 16;          // 2 KiB row blocks per stage
@@ -1023,121 +1025,112 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         constexpr bool PAIRS = NS >= 4 && C::LOADER == LOAD_DMA && !C::BLOCK_SCALE && C::KMAJ == 0 && C::BM * C::BN <= 64 * 128 &&
                                C::KG == 1;
         if constexpr (C::KG == 2) {
-            // Two sets of waves half a turn apart.  Phase s opens with a barrier; behind it the set s & 1 reads the
-            // fragments of stage s and issues the copies of stage s+NS-1, while the other set runs the MFMAs of stage s-1
-            // on the fragments it read one phase earlier.  So the fragment reads and the copies of one set run under the
-            // MFMAs of the other, and a wave about to multiply has nothing else to issue: a stage of copies keeps the
-            // CU's vector memory path busy for about as long as the MFMAs of a stage take, and a wave whose copy
-            // instructions queue there issues no MFMA meanwhile (with every wave copying its share right behind the
-            // barrier, the 16 MFMAs of a stage took twice their 530 cycles).
-            // A set copies whole stages, every other one: 2 * LPT copies per wave and stage.  Stage s is issued in phase
-            // s-NS+1 by the set that reads then; with NS odd that is the set that reads stage s, which waits for it before
-            // the barrier of its own read phase; with NS even it is the other set, which waits before the barrier of its
-            // MFMA phase.  In both cases everything a wave has issued since may stay in flight: (NS-3)/2 or (NS-2)/2
-            // stages.  Behind the barrier of phase s stage s-1 has been read by everybody (a reading wave waits for its
-            // fragments before the next barrier) and its buffer takes stage s+NS-1.  nk + 1 phases, the same barriers for
-            // every wave.  (Touching the lines of later stages with plain loads, so that the copies would find them in
-            // the L2, was tried and made the loop a quarter slower.)
-            // Block scales: a copying wave adds one 4-byte-per-lane copy per stage that brings the a_scale values of 64
-            // tile rows (even waves rows 0 - 63, odd waves rows 64 - 127: the same bytes to the same place from two
-            // waves, so that all waves count alike) to the stage's 512 bytes behind the ring.
-            constexpr int CPS = 2 * C::LPT + (C::BLOCK_SCALE ? 1 : 0);      // copies per stage and copying wave
-            constexpr bool WAIT_AT_READ = (NS & 1) == 1;
-            constexpr int AHEAD = WAIT_AT_READ ? (NS - 3) / 2 : (NS - 2) / 2;   // stages of its own a wave leaves in flight
-            const uint32_t as_voff_k2 = (row0 + 64 * (wave & 1) + lane) * p.as_ms * 4;
-            auto copy_k2 = [&](int kt, int j) {            // copy j (0 .. CPS-1) of stage kt
-                if (j < 2 * C::LPT) {                        // instruction q = wave_q + 4 * j of the stage (see issue_stage)
-                    lds_void *dst = (lds_void *)(smem + (kt % NS) * C::STAGE_BYTES + (wave_q + 4 * j) * 1024);
-                    const bool is_a = j < 2 * LPT_A0;
-                    const uint32_t blk = (wave_q >> 1) + (is_a ? j : j - 2 * LPT_A0) * 2;
-                    const uint32_t soff = blk * 16 * (is_a ? p.lda : p.ldb) + (uint32_t)kt * C::BKB;
-                    if (is_a) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, soff, 0, 0);
-                    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, soff, 0, 0);
-                } else {
-                    lds_void *dst = (lds_void *)(smem + NS * C::STAGE_BYTES + (kt % NS) * 512 + (wave & 1) * 256);
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 4, as_voff_k2, (kbeg + (uint32_t)kt) * p.as_ks * 4, 0, 0);
-                }
-            };
-            auto issue_stage_k2 = [&](int kt) {
+            // Two sets of waves half a turn apart, and four waves that copy.  Phase s opens with a barrier; behind it
+            // the set s & 1 reads the fragments of stage s while the other set runs the MFMAs of stage s-1 on the
+            // fragments it read one phase earlier, and the copying waves issue stage s+NS-1 into the buffer of stage
+            // s-1, which everybody has read (a reading wave waits for its fragments before the next barrier).  So
+            // the fragment reads of one set and the copies run under the MFMAs of the other set, and a wave about
+            // to multiply has nothing else to issue.  That is what the copying waves are for: a stage of copies
+            // keeps the CU's vector memory path busy for 360 - 460 cycles, about as long as the 16 MFMAs of a stage
+            // take (510), and a wave whose copy instructions queue there issues nothing else meanwhile.  With every
+            // wave copying its share right behind the barrier the MFMAs of a stage took twice their time; with the
+            // reading set copying between its fragment reads the read phase took 600 - 700 cycles (the LDS queue and
+            // the memory queue each hold the wave up in turn).
+            // Before the barrier of phase s a copying wave has waited for its half of stage s: everything it
+            // issued since, NS-2 stages, may stay in flight.  nk + 1 phases, the same barriers for every wave.
+            // (Touching the lines of later stages with plain loads, so that the copies would find them in the L2,
+            // was tried and made the loop a quarter slower.)
+            // Block scales: each copying wave adds one 4-byte-per-lane copy per stage that brings the a_scale values
+            // of 64 tile rows (even waves rows 0 - 63, odd waves rows 64 - 127: the same bytes to the same place from
+            // two waves, so that all of them count alike) to the stage's 512 bytes behind the ring.
+            constexpr int NPC = C::NLOAD / C::NPROD;                        // operand copies per stage and copying wave
+            constexpr int CPS = NPC + (C::BLOCK_SCALE ? 1 : 0);
+            static_assert(C::NPROD == 4 && C::NLOAD % 4 == 0 && C::RBA % 2 == 0 && (NS - 2) * CPS <= 63,
+                          "copying waves: an even share each, copies in flight within the 6-bit counter");
+            if (kg == 2) {
+                // instruction q = pw + 4 * j of the stage (see issue_stage; pw = 0 .. 3, q & 1 = wave & 1): rows
+                // 8 * (q & 1) .. + 7 of row block q >> 1, the first RBA row blocks are A's
+                const int pw = wave & 3;
+                const uint32_t as_voff_k2 = (row0 + 64 * (wave & 1) + lane) * p.as_ms * 4;
+                auto issue_stage_k2 = [&](int kt) {
+                    char *stage = smem + (kt % NS) * C::STAGE_BYTES + pw * 1024;
 #pragma unroll
-                for (int j = 0; j < CPS; ++j) copy_k2(kt, j);
-            };
-            v4i fa[C::TM][2], fb[C::TN][2];
-            auto open_phase = [&](int ph, bool own_read) {
-                if (own_read == WAIT_AT_READ) {
-                    // the newest stage this wave can have issued: in its read phase ph-2 or ph-1
-                    if (ph + NS - (WAIT_AT_READ ? 3 : 2) < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm(AHEAD * CPS));
-                    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
-                }
-                ring_barrier();
-            };
-            // The read phase: fragment reads and copies in turn, two reads to a copy.  Sixteen 1 KiB reads of each of the
-            // four waves fill the LDS queue and the copies fill the vector memory queue; either kind issued in one run
-            // holds the wave for as long as its unit takes to drain (about 380 and 360 cycles), taken in turn the two
-            // units drain side by side.
-            auto read_stage = [&](int mine, int refill, auto with_copies) {
-                constexpr bool COPIES = decltype(with_copies)::value;
-                if constexpr (C::BLOCK_SCALE) {
-                    const char *sc = smem + NS * C::STAGE_BYTES + (mine % NS) * 512 + (wm * C::WM + (lane & 15)) * 4;
-#pragma unroll
-                    for (int a = 0; a < C::TM; ++a) as_cur[a] = *(const float *)(sc + a * 64);
-                    const uint32_t kb = kbeg + (uint32_t)mine;
-#pragma unroll
-                    for (int j = 0; j < NBS; ++j)
-                        bs_cur[j] = p.bs[__builtin_amdgcn_readfirstlane(bs_off[j] + kb * p.bs_ks)];
-                }
-                const char *st = smem + (mine % NS) * C::STAGE_BYTES;
-                constexpr int NREAD = 2 * (C::TM + C::TN);
-#pragma unroll
-                for (int i = 0; i < NREAD; ++i) {
-                    if (i < 2 * C::TM) fa[i / 2][i % 2] = frag_a(st, i / 2, i % 2);
-                    else fb[(i - 2 * C::TM) / 2][i % 2] = frag_b(st, (i - 2 * C::TM) / 2, i % 2);
-                    if constexpr (COPIES) {
-                        if (i % 2 == 1) {
-                            __builtin_amdgcn_sched_barrier(0);
-                            if (i / 2 < CPS) copy_k2(refill, i / 2);
-                            __builtin_amdgcn_sched_barrier(0);
-                        }
+                    for (int j = 0; j < NPC; ++j) {
+                        lds_void *dst = (lds_void *)(stage + j * 4096);
+                        const uint32_t blk = (pw >> 1) + 2 * j;
+                        if (2 * j < C::RBA)
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, blk * 16 * p.lda + (uint32_t)kt * C::BKB, 0, 0);
+                        else
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, (blk - C::RBA) * 16 * p.ldb + (uint32_t)kt * C::BKB, 0, 0);
                     }
-                }
-                if constexpr (COPIES) {
+                    if constexpr (C::BLOCK_SCALE) {
+                        lds_void *dst = (lds_void *)(smem + NS * C::STAGE_BYTES + (kt % NS) * 512 + (wave & 1) * 256);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 4, as_voff_k2, (kbeg + (uint32_t)kt) * p.as_ks * 4, 0, 0);
+                    }
+                };
 #pragma unroll
-                    for (int j = NREAD / 2; j < CPS; ++j) copy_k2(refill, j);
+                for (int j = 0; j < NS - 1; ++j)
+                    if (j < nk) issue_stage_k2(j);
+                for (int ph = 0; ph <= nk; ++ph) {
+                    if (ph + NS - 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * CPS));
+                    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
+                    ring_barrier();
+                    if (ph + NS - 1 < nk) issue_stage_k2(ph + NS - 1);
                 }
-            };
-            auto mfma_stage = [&]() {
+            } else {
+                v4i fa[C::TM][2], fb[C::TN][2];
+                auto read_stage = [&](int mine) {
+                    if constexpr (C::BLOCK_SCALE) {
+                        const char *sc = smem + NS * C::STAGE_BYTES + (mine % NS) * 512 + (wm * C::WM + (lane & 15)) * 4;
 #pragma unroll
-                for (int b = 0; b < C::TN; ++b)
+                        for (int a = 0; a < C::TM; ++a) as_cur[a] = *(const float *)(sc + a * 64);
+                        const uint32_t kb = kbeg + (uint32_t)mine;
+#pragma unroll
+                        for (int j = 0; j < NBS; ++j)
+                            bs_cur[j] = p.bs[__builtin_amdgcn_readfirstlane(bs_off[j] + kb * p.bs_ks)];
+                    }
+                    const char *st = smem + (mine % NS) * C::STAGE_BYTES;
 #pragma unroll
                     for (int a = 0; a < C::TM; ++a) {
-                        if constexpr (C::BLOCK_SCALE) {
-                            // P * (as * bs), then accumulate (hip_mix_gemm_kernel.cpp:241 has (P * as) * bs: the
-                            // factor formed first is one multiply per row and K block instead of four per MFMA)
-                            const v4f part = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                            const float f = as_cur[a] * bs_cur[(b * 16) / 128];
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) acc[a][b][r] += part[r] * f;
-                        } else {
-                            acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
-                        }
+                        fa[a][0] = frag_a(st, a, 0);
+                        fa[a][1] = frag_a(st, a, 1);
                     }
-            };
 #pragma unroll
-            for (int j = 0; j < NS - 1; ++j)
-                if (j < nk && ((j + NS - 1) & 1) == kg) issue_stage_k2(j);
-            int ph = 0;
-            if (kg == 1) {                       // phase 0 of the second set: nothing to multiply yet
-                open_phase(0, false);
-                ph = 1;
-            }
-            for (; ph <= nk; ph += 2) {
-                open_phase(ph, true);
-                if (ph + NS - 1 < nk) read_stage(ph, ph + NS - 1, std::true_type{});
-                else if (ph < nk) read_stage(ph, 0, std::false_type{});
-                __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());   // reads done before the buffer may be refilled
-                if (ph + 1 <= nk) {
-                    open_phase(ph + 1, false);
-                    mfma_stage();
+                    for (int b = 0; b < C::TN; ++b) {
+                        fb[b][0] = frag_b(st, b, 0);
+                        fb[b][1] = frag_b(st, b, 1);
+                    }
+                    __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());   // reads done before the buffer may be refilled
+                };
+                auto mfma_stage = [&]() {
+#pragma unroll
+                    for (int b = 0; b < C::TN; ++b)
+#pragma unroll
+                        for (int a = 0; a < C::TM; ++a) {
+                            if constexpr (C::BLOCK_SCALE) {
+                                // P * (as * bs), then accumulate (hip_mix_gemm_kernel.cpp:241 has (P * as) * bs: the
+                                // factor formed first is one multiply per row and K block instead of four per MFMA)
+                                const v4f part = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                                const float f = as_cur[a] * bs_cur[(b * 16) / 128];
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) acc[a][b][r] += part[r] * f;
+                            } else {
+                                acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                            }
+                        }
+                };
+                int ph = 0;
+                if (kg == 1) {                       // phase 0 of the second set: nothing to multiply yet
+                    ring_barrier();
+                    ph = 1;
+                }
+                for (; ph <= nk; ph += 2) {
+                    ring_barrier();
+                    if (ph < nk) read_stage(ph);
+                    if (ph + 1 <= nk) {
+                        ring_barrier();
+                        mfma_stage();
+                    }
                 }
             }
         } else if constexpr (PAIRS) {
@@ -1295,7 +1288,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 for (int b = 0; b < C::TN; ++b) *(acc_t *)(part + (a * C::TN + b) * 1024) = acc[a][b];
         }
         __syncthreads();
-        if (kg == 1) return;
+        if (kg >= 1) return;                               // set 1 and the copying waves are done
 #pragma unroll
         for (int a = 0; a < C::TM; ++a)
 #pragma unroll

@@ -62,7 +62,7 @@ struct Context {
 #endif
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
-    long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes
+    long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes; 2: never
     std::string last_config;
 };
 
@@ -245,10 +245,10 @@ bool mfma_shape_ok(const NtProblem &q) {
 // workgroup alone on its CU runs its steps faster, and a K split pays a second launch plus the traffic of the
 // partial planes.  The times per 128-byte K step were read off a sweep of every variant over square and oblong
 // shapes from 1024 to 8192 (fp8 and bf16 agree per step; block scales have figures of their own): 1.25 us for the
-// 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.52 us for the 128 x 128
-// row with two K groups (one per CU: it only wins where there are no more tiles than CUs), 0.52 us for 64 x 128 and
-// 0.36 us for its row with two K groups (graph replays of 384 / 512 x 4096 x 4096 and 1024 x 2048 x 7168), 0.39 us for
-// 128 x 32.  A K split adds 4 us and the partial planes at 3 TB/s.
+// 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.43 us for the 128 x 128
+// row with two K groups (one per CU: it only wins where there are no more tiles than CUs; 2048 x 2048 x 2048 / 8192
+// 12.1 / 32.5 us), 0.52 us for 64 x 128 and 0.27 us for its row with two K groups (512 x 4096 x 4096 13.5 us, two
+// rounds of 64 steps 44 us), 0.39 us for 128 x 32.  A K split adds 4 us and the partial planes at 3 TB/s.
 //
 // M <= 64 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
 // workgroup, else the shortest tile that covers the rows; narrow tiles instead of a K split.  (65 .. 128 rows go
@@ -264,11 +264,11 @@ struct TileModel {
     double blk_shared, blk_alone;
 };
 // (block scales, graph replays: 256 x 256 2048 x 4608 x 7168 77 us, 1536 x 7168 x 2048 27.6; 128 x 128 1024 x 7168 x 2048 25.9,
-// 1024 x 4608 x 7168 75.0; 64 x 128 1024 x 4608 x 7168 69.9, 512 x 4608 x 7168 47.8; K groups 512 x 7168 x 2048 16.8 and 12.9 for
-// 256 rows; 128 x 32 256 x 7168 x 2048 12.9)
+// 1024 x 4608 x 7168 75.0; 64 x 128 1024 x 4608 x 7168 69.9, 512 x 4608 x 7168 47.8; K groups 128 x 128 2048 x 2048 x 2048 /
+// 8192 14 / 43, 64 x 128 512 x 4096 x 4096 18; 128 x 32 256 x 7168 x 2048 12.9)
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.40, 1.10},
-                                 {128, 128, 1, 0.52, 0.52, 3.0, true, 1, 0.92, 0.92},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
-                                 {64, 128, 1, 0.36, 0.36, 2.5, true, 1, 0.72, 0.72},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
+                                 {128, 128, 1, 0.43, 0.43, 4.5, true, 1, 0.60, 0.60},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
+                                 {64, 128, 1, 0.27, 0.27, 4.5, true, 1, 0.40, 0.40},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
 // rows with two K groups: eight waves on a tile that otherwise has four (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 
@@ -393,9 +393,10 @@ int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps
 
 // Should the problem run with these operands read K-major, as they are stored (strides between k rows given)?
 // Yes when the shape fits and the estimate for the K-major family (simple pipeline, two stages, transposing reads:
-// a fifth slower per step) beats the K-contiguous kernel plus the transpose launch in front of it (about 5 us and
-// the matrices read and written at about 5 TB/s).  Large shapes keep the transposes and the
-// pipelined 256 x 256 tile; small and mid-size ones save the launches.
+// 15 % on top of the estimate) beats the K-contiguous kernel plus the transpose launches in front of it (4 us per
+// operand and the matrix read and written at 5.5 TB/s; block scales 2048^3 in the reference's layout: 23.3 us as
+// stored, 29.3 us behind two transposes; 1024 x 4096 x 4096: 39.9 against 37.2).  Large shapes keep the transposes
+// and the pipelined 256 x 256 tile; small and mid-size ones save the launches.
 bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes) {
     if (!g_ctx.kmajor) return false;
     q.kmaj = kmaj;
@@ -406,6 +407,7 @@ bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes
     const Variant *tab = table_for(q.arith, q.block, 0, &count), *tab_km = table_for(q.arith, q.block, kmaj, &count_km);
     if (!tab || !tab_km || count != count_km) return false;
     if (g_ctx.force_config >= 0 && g_ctx.force_config < count) return true;    // forced rows exist in every family
+    if (g_ctx.kmajor == 2) return true;                                        // measurements: as stored wherever possible
     const size_t ksteps = q.Kbytes / 128;
     const bool may_split = q.split_k == 0;
     uint32_t ns = 0;
@@ -414,10 +416,10 @@ bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes
     if (q.M > 128 && choose_by_cost(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, may_split, &ns, &t_nt) < 0)
         return false;
     const double kbytes = (double)q.Kbytes;         // K * element size
-    t_nt += 5.0;                                     // one launch transposes whatever has to be transposed
-    if (kmaj & 1) t_nt += 2.0 * (double)q.M * kbytes / 5.0e6;
-    if (kmaj & 2) t_nt += 2.0 * (double)q.N * kbytes / 5.0e6;
-    return 1.2 * t_km <= t_nt;
+    t_nt += 1.0;                                     // a transpose launch per operand: 4 us and the matrix read and written
+    if (kmaj & 1) t_nt += 4.0 + 2.0 * (double)q.M * kbytes / 5.5e6;
+    if (kmaj & 2) t_nt += 4.0 + 2.0 * (double)q.N * kbytes / 5.5e6;
+    return 1.15 * t_km <= t_nt;
 }
 
 struct Plan {
