@@ -1036,7 +1036,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // wave copying its share right behind the barrier the MFMAs of a stage took twice their time; with the
             // reading set copying between its fragment reads the read phase took 600 - 700 cycles (the LDS queue and
             // the memory queue each hold the wave up in turn).
-            // Before the barrier of phase s a copying wave has waited for its half of stage s: everything it
+            // Before the barrier of phase s a copying wave has waited for its quarter of stage s: everything it
             // issued since, NS-2 stages, may stay in flight.  nk + 1 phases, the same barriers for every wave.
             // (Touching the lines of later stages with plain loads, so that the copies would find them in the L2,
             // was tried and made the loop a quarter slower.)
