@@ -1,0 +1,61 @@
+"""The rows with two K groups per workgroup (two sets of computing waves half a turn apart, copying waves beside them):
+every number of K steps from one up to past twice the ring, so that the first phases (nothing to multiply yet), the
+last ones (nothing left to read or copy) and every ring position are hit; with and without a K split; on ragged
+tiles.  Small integers (and power-of-two block scales) sum exactly in fp32 and int32, so the results must equal the
+CPU oracle bit for bit: a stage read too early, a buffer refilled too soon or a step left out cannot hide."""
+import numpy as np
+import pytest
+import torch
+
+import qgemm_amd as Q
+from oracle import cpu_ref as R
+from tests.util import dev, fp8_tensor, host, say, scalar
+
+pytestmark = pytest.mark.gpu
+ROWS = {"128x128_w2x2_k2": 16, "64x128_w1x4_k2": 17}       # rows of the variant table
+
+
+@pytest.fixture(autouse=True)
+def _reset_options():
+    yield
+    for k, v in (("force_config", -1), ("force_split", 0)):
+        Q.set_option(k, v)
+
+
+@pytest.mark.parametrize("row", sorted(ROWS))
+@pytest.mark.parametrize("fam", ["f8", "f8_block", "i8", "bf16"])
+def test_every_number_of_k_steps(row, fam):
+    M, N = 200, 328                                          # ragged in both directions, several tiles
+    for ksteps in range(1, 14):
+        for split in ((0, 2) if ksteps >= 4 else (0,)):
+            K = ksteps * (64 if fam == "bf16" else 128)
+            say("k groups", row, fam, (M, N, K), "split", split)
+            Q.set_option("force_config", ROWS[row])
+            Q.set_option("force_split", split if split else 1)
+            rng = np.random.default_rng(100 * ksteps + split)
+            a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+            b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+            if fam == "i8":
+                c = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+                Q.int8_mm(dev(a.astype(np.int8)), dev(b.astype(np.int8)), scalar(1), scalar(1), c)
+                ref = R.gemm_i8_i32(a.astype(np.int8), b.astype(np.int8))
+            elif fam == "bf16":
+                c = torch.full((M, N), -7.0, dtype=torch.float32, device="cuda")
+                Q.gemm(dev(a).bfloat16(), dev(b).bfloat16(), c, "nk")
+                ref = R.gemm_f32acc(a, b)
+            elif fam == "f8":
+                c = torch.full((M, N), -7.0, dtype=torch.float32, device="cuda")
+                Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), scalar(1), scalar(1), c, M, N, K,
+                              Q.SCALE_PER_MATRIX)
+                ref = R.gemm_f32acc(a, b)
+            else:
+                as_ = (2.0 ** rng.integers(-3, 4, size=(M, ksteps))).astype(np.float32)
+                bs = (2.0 ** rng.integers(-3, 4, size=((N + 127) // 128, ksteps))).astype(np.float32)
+                c = torch.full((M, N), -7.0, dtype=torch.float32, device="cuda")
+                Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K,
+                              Q.SCALE_BLOCK128)
+                ref = R.gemm_fp8_block(a, b, as_, bs)
+            name = Q.last_config()
+            assert name.startswith(row), name
+            assert ("splitk" in name) == (split > 1), name
+            assert np.array_equal(host(c), ref), (name, ksteps, split)
