@@ -181,6 +181,46 @@ def vendor_sweep(Q, torch, dev):
     return rows
 
 
+def one_shape(Q, torch, dev, spec, launches):
+    """`--shape fp8:2048x2048x8192` (fp8 | fp8block | int8 | bf16 | fp16): this library alone on one shape, `launches`
+    calls from a replayed graph after as many to warm up; for profiling a single kernel, or for trying a shape."""
+    fam, dims = spec.split(":")
+    M, N, K = (int(x) for x in dims.lower().split("x"))
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    if fam == "fp8":
+        a, sa = _quant_fp8(torch.randn(M, K, device=dev)); b, sb = _quant_fp8(torch.randn(N, K, device=dev))
+        fn = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)
+    elif fam == "fp8block":
+        a, _ = _quant_fp8(torch.randn(M, K, device=dev)); b, _ = _quant_fp8(torch.randn(N, K, device=dev))
+        sa = (torch.rand(M, K // 128, device=dev) + 0.5) / 448; sb = (torch.rand((N + 127) // 128, K // 128, device=dev) + 0.5) / 448
+        fn = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_BLOCK128)
+    elif fam == "int8":
+        a, sa = _quant_i8(torch.randn(M, K, device=dev)); b, sb = _quant_i8(torch.randn(N, K, device=dev))
+        fn = lambda: Q.int8_mm(a, b, sa, sb, c)
+    elif fam in ("bf16", "fp16"):
+        dt = torch.bfloat16 if fam == "bf16" else torch.float16
+        a = torch.randn(M, K, device=dev).to(dt); b = torch.randn(N, K, device=dev).to(dt)
+        c = torch.empty(M, N, dtype=dt, device=dev)
+        fn = lambda: Q.gemm(a, b, c, "nk")
+    else:
+        raise SystemExit("bench.py --shape: type must be fp8, fp8block, int8, bf16 or fp16")
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(launches):
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(); g.replay(); e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / launches
+    return {"type": fam, "M": M, "N": N, "K": K, "kernel": Q.last_config(), "launches": launches, "us_per_launch": round(us, 2),
+            "tflops": round(2.0 * M * N * K / us / 1e6, 1)}
+
+
 def skinny_probe(Q, torch, dev):
     """Where a launch of the skinny-M kernel spends its time (config 5 shapes, fp8):
       * graph-replay time per launch with B resident against the number of 32-column strips (= workgroups), K and
@@ -248,6 +288,9 @@ def main():
     ap.add_argument("--vendor-sweep", action="store_true",
                     help="only time this library against the vendor library (torch.matmul, torch._scaled_mm, "
                          "torch._int_mm) over a list of shapes, interleaved, print one JSON line and exit")
+    ap.add_argument("--shape", default="",
+                    help="only run this library on one shape, e.g. fp8:2048x2048x8192 (fp8 | fp8block | int8 | bf16 | fp16), "
+                         "--steps launches from a replayed graph; print one JSON line and exit")
     ap.add_argument("--skinny-probe", action="store_true",
                     help="only probe where the skinny-M kernel (config 5) spends its time, print one JSON line and exit")
     args = ap.parse_args()
@@ -271,6 +314,9 @@ def main():
         return 0
     torch.manual_seed(42)                 # seed of the reference harness, tests/includes/test_config.h:64
     dev = "cuda:0"
+    if args.shape:
+        print(json.dumps({"shape": one_shape(Q, torch, dev, args.shape, max(1, min(args.steps, 200)))}))
+        return 0
     if args.vendor_sweep:
         print(json.dumps({"vendor_sweep": vendor_sweep(Q, torch, dev)}))
         return 0
