@@ -1103,21 +1103,40 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());   // reads done before the buffer may be refilled
                 };
                 auto mfma_stage = [&]() {
+                    if constexpr (C::BLOCK_SCALE) {
+                        // P * (as * bs), then accumulate (hip_mix_gemm_kernel.cpp:241 has (P * as) * bs: the factor
+                        // formed first is one multiply per row and K block instead of four per MFMA).  Each MFMA starts
+                        // from zero; its partial product is folded into the running sum one MFMA later, so that the
+                        // four FMAs of a tile run under the MFMA of the next (straight after its own MFMA they would
+                        // wait for it, and the next MFMA for them: 60 cycles a tile instead of 32).
+                        constexpr int NT = C::TM * C::TN;
+                        float f[C::TM][NBS];
 #pragma unroll
-                    for (int b = 0; b < C::TN; ++b)
+                        for (int a = 0; a < C::TM; ++a)
 #pragma unroll
-                        for (int a = 0; a < C::TM; ++a) {
-                            if constexpr (C::BLOCK_SCALE) {
-                                // P * (as * bs), then accumulate (hip_mix_gemm_kernel.cpp:241 has (P * as) * bs: the
-                                // factor formed first is one multiply per row and K block instead of four per MFMA)
-                                const v4f part = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                                const float f = as_cur[a] * bs_cur[(b * 16) / 128];
+                            for (int j = 0; j < NBS; ++j) f[a][j] = as_cur[a] * bs_cur[j];
+                        v4f part[2];
 #pragma unroll
-                                for (int r = 0; r < 4; ++r) acc[a][b][r] += part[r] * f;
-                            } else {
-                                acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                        for (int i = 0; i <= NT; ++i) {
+                            if (i < NT) {
+                                const int a = i % C::TM, b = i / C::TM;
+                                part[i & 1] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
                             }
+                            __builtin_amdgcn_sched_barrier(0);       // MFMA i first, the FMAs of tile i-1 under it
+                            if (i > 0) {
+                                const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f[pa][(pb * 16) / 128];
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
                         }
+                    } else {
+#pragma unroll
+                        for (int b = 0; b < C::TN; ++b)
+#pragma unroll
+                            for (int a = 0; a < C::TM; ++a)
+                                acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
+                    }
                 };
                 int ph = 0;
                 if (kg == 1) {                       // phase 0 of the second set: nothing to multiply yet
@@ -1219,6 +1238,13 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 fa[a][0] = frag_a(stage, a, 0);
                 fa[a][1] = frag_a(stage, a, 1);
             }
+            v4f part[2];                                     // block scales: the partial products of two tiles
+            auto fold_tile = [&](int i) {
+                const int pa = i % C::TM, pb = i / C::TM;
+                const float f = as_cur[pa] * bs_cur[(pb * 16) / 128];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[i & 1][r] * f;
+            };
             v4i fball[READS_FIRST ? C::TN : 1][2];
             if constexpr (READS_FIRST) {
 #pragma unroll
@@ -1242,16 +1268,17 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 for (int a = 0; a < C::TM; ++a) {
                     if constexpr (C::BLOCK_SCALE) {
                         // P * (as * bs), then accumulate (hip_mix_gemm_kernel.cpp:241 has (P * as) * bs: the factor
-                        // formed first is one multiply per row and K block instead of four per MFMA)
-                        const v4f part = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                        const float f = as_cur[a] * bs_cur[(b * 16) / 128];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[a][b][r] += part[r] * f;
+                        // formed first is one multiply per row and K block instead of four per MFMA), one MFMA behind:
+                        // the four FMAs of a tile go behind the MFMA of the next tile and run under it
+                        const int i = b * C::TM + a;
+                        part[i & 1] = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                        if (i > 0) fold_tile(i - 1);
                     } else {
                         acc[a][b] = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], acc[a][b]);
                     }
                 }
             }
+            if constexpr (C::BLOCK_SCALE) fold_tile(C::TM * C::TN - 1);
             if constexpr (C::LOADER == LOAD_VGPR) {
                 // the other stage was last read in iteration kt-1, which every wave left before this one began
                 if (kt + 1 < nk) commit_stage(kt + 1);

@@ -192,14 +192,21 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
             for (int a = 0; a < C::TM; ++a)
                 f[a] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((((16 * a) & 63) + (lane & 15)) * 4,
                                                                                 as_cur[s][(16 * a) / 64])) * bs_cur[s];
+            // one MFMA behind: the four FMAs of a tile go behind the MFMA of the next tile and run under it (straight
+            // after their own MFMA they would wait for it, and the next MFMA for them)
+            v4f part[2];
 #pragma unroll
-            for (int b = 0; b < C::TN; ++b)
-#pragma unroll
-                for (int a = 0; a < C::TM; ++a) {
-                    const v4f part = mma128<C::ARITH>(fb[s][b][0], fb[s][b][1], fa[s][a][0], fa[s][a][1], v4f{0, 0, 0, 0});
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[a][b][r] += part[r] * f[a];
+            for (int i = 0; i <= C::TM * C::TN; ++i) {
+                if (i < C::TM * C::TN) {
+                    const int a = i % C::TM, b = i / C::TM;
+                    part[i & 1] = mma128<C::ARITH>(fb[s][b][0], fb[s][b][1], fa[s][a][0], fa[s][a][1], v4f{0, 0, 0, 0});
                 }
+                if (i > 0) {
+                    const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f[pa];
+                }
+            }
         } else {
 #pragma unroll
             for (int b = 0; b < C::TN; ++b)

@@ -266,8 +266,8 @@ struct TileModel {
 // (block scales, graph replays: 256 x 256 2048 x 4608 x 7168 77 us, 1536 x 7168 x 2048 27.6; 128 x 128 1024 x 7168 x 2048 25.9,
 // 1024 x 4608 x 7168 75.0; 64 x 128 1024 x 4608 x 7168 69.9, 512 x 4608 x 7168 47.8; K groups 128 x 128 2048 x 2048 x 2048 /
 // 8192 14 / 43, 64 x 128 512 x 4096 x 4096 18; 128 x 32 256 x 7168 x 2048 12.9)
-const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.40, 1.10},
-                                 {128, 128, 1, 0.43, 0.43, 4.5, true, 1, 0.60, 0.60},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
+const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.32, 1.04},
+                                 {128, 128, 1, 0.43, 0.43, 4.5, true, 1, 0.55, 0.55},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
                                  {64, 128, 1, 0.27, 0.27, 4.5, true, 1, 0.40, 0.40},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
 // rows with two K groups: eight waves on a tile that otherwise has four (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
