@@ -98,9 +98,9 @@ static const Variant kTable[] = {
     ROW("128x32_w4x1_dma", 128, 32, 4, 1, LOAD_DMA, true),
     ROW("64x32_w4x1_dma", 64, 32, 4, 1, LOAD_DMA, true),
     ROW("16x32_w1x2_dma", 16, 32, 1, 2, LOAD_DMA, true),
-    // 128 x 128 with eight waves in two K groups (GemmCfg::KG) and five stages (160 KiB, one workgroup per CU; four
-    // with block scales, whose a_scale values take 2 KiB behind the ring): for shapes with no more tiles than CUs,
-    // where the two-stage row above would sit alone on its CU
+    // 128 x 128 with eight computing waves in two K groups and four copying waves (GemmCfg::KG), five stages (160 KiB,
+    // one workgroup per CU; four with block scales, whose a_scale values take 2 KiB behind the ring): for shapes with
+    // no more tiles than CUs, where the two-stage row above would sit alone on its CU
 #if INST_KMAJ      // (no K-major form: alias, so indices agree across families)
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #else

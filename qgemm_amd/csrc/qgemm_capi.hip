@@ -269,7 +269,7 @@ struct TileModel {
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.32, 1.04},
                                  {128, 128, 1, 0.43, 0.43, 4.5, true, 1, 0.55, 0.55},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
                                  {64, 128, 1, 0.27, 0.27, 4.5, true, 1, 0.40, 0.40},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
-// rows with two K groups: eight waves on a tile that otherwise has four (one workgroup per CU)
+// rows with two K groups: two sets of computing waves on a tile that otherwise has one (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 
 int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus, bool may_split,
