@@ -101,19 +101,16 @@ static const Variant kTable[] = {
     // 128 x 128 with eight computing waves in two K groups and four copying waves (GemmCfg::KG), five stages (160 KiB,
     // one workgroup per CU; four with block scales, whose a_scale values take 2 KiB behind the ring): for shapes with
     // no more tiles than CUs, where the two-stage row above would sit alone on its CU
-#if INST_KMAJ      // (no K-major form: alias, so indices agree across families)
-    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
-#else
-    row_of<true, GemmCfg<INST_ARITH, (bool)INST_BLOCK, 128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, INST_BLOCK ? 4 : 5, 2>,
+    // (K-major families too: the waves that read the tile with the transposing LDS reads have no copies in flight)
+    row_of<kmajor_can(128, 128, 4, PIPE_SIMPLE),
+           GemmCfg<INST_ARITH, (bool)INST_BLOCK, 128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE, 0, false, INST_KMAJ, INST_BLOCK ? 4 : 5, 2>,
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("128x128_w2x2_k2", true),
-#endif
-    // the same for the 64 x 128 tile, with six stages (two turns of copies in flight)
-#if INST_KMAJ
-    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
-#else
-    row_of<true, GemmCfg<INST_ARITH, (bool)INST_BLOCK, 64, 128, 1, 4, LOAD_DMA, PIPE_SIMPLE, 0, false, 0, 6, 2>,
+    // the same for the 64 x 128 tile, with six stages
+    row_of<kmajor_can(64, 128, 4, PIPE_SIMPLE),
+           GemmCfg<INST_ARITH, (bool)INST_BLOCK, kmajor_can(64, 128, 4, PIPE_SIMPLE) ? 64 : 128, 128, kmajor_can(64, 128, 4, PIPE_SIMPLE) ? 1 : 2,
+                   kmajor_can(64, 128, 4, PIPE_SIMPLE) ? 4 : 2, LOAD_DMA, PIPE_SIMPLE, 0, false, INST_KMAJ,
+                   kmajor_can(64, 128, 4, PIPE_SIMPLE) ? 6 : (INST_BLOCK ? 4 : 5), 2>,
            CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("64x128_w1x4_k2", true),
-#endif
     // skinny M (gemm_skinny.cuh): the K split inside the workgroup, no staging, no barrier in the K loop
 #if INST_KMAJ      // (no K-major form: aliases, so indices agree across families)
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),

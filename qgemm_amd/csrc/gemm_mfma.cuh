@@ -160,10 +160,10 @@ struct GemmCfg {
     // wave's own count of copies in flight stays exact (a register load among them makes the compiler wait for all).
     static constexpr int SCALE_LDS = (BLOCK_SCALE_ && KGROUPS_ == 2) ? NSTAGE * 512 : 0;
     static constexpr int LDS_BYTES = (A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES) + SCALE_LDS;
-    static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && (!BLOCK_SCALE || KGROUPS_ == 2) && KMAJ_ == 0 &&
-                                   STAGES_ >= 2 && STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
+    static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && (!BLOCK_SCALE || KGROUPS_ == 2) &&
+                                   (KMAJ_ == 0 || KGROUPS_ == 2) && STAGES_ >= 2 && STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
                   "explicit stage count: simple pipeline, DMA loader, within LDS and the 6-bit counter");
-    static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && KMAJ_ == 0 &&
+    static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA &&
                                     NSTAGE >= 4 && (!BLOCK_SCALE_ || (BM_ <= 128 && BN_ <= 128))),
                   "K groups: simple pipeline, DMA loader, at least four stages");
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
@@ -185,6 +185,8 @@ struct GemmCfg {
     // The compiler makes every transposing LDS read wait for all global->LDS copies in flight (vmcnt(0)): it cannot
     // tell that they target another buffer.  The simple pipeline issues the next stage's copies behind the reads
     // of a step, so nothing is in flight there; the pipelined schedules live on copies in flight and would stall.
+    // (The rows with two K groups keep a deep ring all the same: their copies are issued by waves of their own, and
+    // the waves that read have none in flight.)
     static_assert(KMAJ == 0 || PIPE == PIPE_SIMPLE, "K-major tiles: simple pipeline only");
     static_assert(!ASK_ || (BLOCK_SCALE_ && PIPE_ == PIPE_SOLO), "K-contiguous a_scale: block scales, solo pipeline");
 };
@@ -1037,7 +1039,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // reading set copying between its fragment reads the read phase took 600 - 700 cycles (the LDS queue and
             // the memory queue each hold the wave up in turn).
             // Before the barrier of phase s a copying wave has waited for its quarter of stage s: everything it
-            // issued since, NS-2 stages, may stay in flight.  nk + 1 phases, the same barriers for every wave.
+            // issued since, NS-2 stages, may stay in flight.  nk + 1 phases, the same barriers for every wave (bare
+            // barriers also for K-major tiles: no wave that reads LDS here has copies in flight).
             // (Touching the lines of later stages with plain loads, so that the copies would find them in the L2,
             // was tried and made the loop a quarter slower.)
             // Block scales: each copying wave adds one 4-byte-per-lane copy per stage that brings the a_scale values
@@ -1052,6 +1055,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // 8 * (q & 1) .. + 7 of row block q >> 1, the first RBA row blocks are A's
                 const int pw = wave & 3;
                 const uint32_t as_voff_k2 = (row0 + 64 * (wave & 1) + lane) * p.as_ms * 4;
+                // scalar offset of row block blk of an operand at K step kt: as load_soff
+                auto soff_k2 = [&](bool kmajor, uint32_t blk, uint32_t ld, int kt) -> uint32_t {
+                    constexpr uint32_t BPP = C::KE / 16;                        // row blocks per panel
+                    if (kmajor) return ((uint32_t)kt * C::KE + (blk % BPP) * 16) * ld + (blk / BPP) * 128;
+                    return blk * 16 * ld + (uint32_t)kt * C::BKB;
+                };
                 auto issue_stage_k2 = [&](int kt) {
                     char *stage = smem + (kt % NS) * C::STAGE_BYTES + pw * 1024;
 #pragma unroll
@@ -1059,9 +1068,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         lds_void *dst = (lds_void *)(stage + j * 4096);
                         const uint32_t blk = (pw >> 1) + 2 * j;
                         if (2 * j < C::RBA)
-                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, blk * 16 * p.lda + (uint32_t)kt * C::BKB, 0, 0);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, soff_k2(C::KMA, blk, p.lda, kt), 0, 0);
                         else
-                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, (blk - C::RBA) * 16 * p.ldb + (uint32_t)kt * C::BKB, 0, 0);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 0);
                     }
                     if constexpr (C::BLOCK_SCALE) {
                         lds_void *dst = (lds_void *)(smem + NS * C::STAGE_BYTES + (kt % NS) * 512 + (wave & 1) * 256);
@@ -1074,7 +1083,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 for (int ph = 0; ph <= nk; ++ph) {
                     if (ph + NS - 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * CPS));
                     else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
-                    ring_barrier();
+                    phase_barrier();
                     if (ph + NS - 1 < nk) issue_stage_k2(ph + NS - 1);
                 }
             } else {
@@ -1140,14 +1149,14 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 };
                 int ph = 0;
                 if (kg == 1) {                       // phase 0 of the second set: nothing to multiply yet
-                    ring_barrier();
+                    phase_barrier();
                     ph = 1;
                 }
                 for (; ph <= nk; ph += 2) {
-                    ring_barrier();
+                    phase_barrier();
                     if (ph < nk) read_stage(ph);
                     if (ph + 1 <= nk) {
-                        ring_barrier();
+                        phase_barrier();
                         mfma_stage();
                     }
                 }

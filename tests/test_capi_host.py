@@ -140,9 +140,10 @@ def test_plan_names_the_kernel_without_a_device():
     finally:
         Q.set_option("row_split", 1)
     # operands stored K-major: read as stored where that is cheaper than transposing, else transposed first
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 2048, 2048, 2048) == "128x128_w2x2_dma_tn"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 2048, 2048, 2048) == "128x128_w2x2_k2_tn"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 4096, 2048, 2048) == "128x128_w2x2_dma_tn"
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 6144, 4608, 7168) == "transpose+256x256_w2x4_solo8"
-    assert plan(Q.DT_BF16, 0, 2, 1024, 1024, 1024) == "64x128_w1x4_dma_nn"
+    assert plan(Q.DT_BF16, 0, 2, 1024, 1024, 1024) == "64x128_w1x4_k2_nn"
     assert plan(Q.DT_BF16, 0, 2, 8192, 8192, 8192) == "transpose+256x256_w2x2_solo"
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 2, 1024, 1024, 1024).startswith("transpose+")   # no K-major int8 family
     # K not a multiple of 128 bytes: the any-shape kernel
