@@ -18,7 +18,7 @@ ROWS = {"128x128_w2x2_k2": 16, "64x128_w1x4_k2": 17}       # rows of the variant
 @pytest.fixture(autouse=True)
 def _reset_options():
     yield
-    for k, v in (("force_config", -1), ("force_split", 0)):
+    for k, v in (("force_config", -1), ("force_split", 0), ("kmajor", 1)):
         Q.set_option(k, v)
 
 
@@ -59,3 +59,35 @@ def test_every_number_of_k_steps(row, fam):
             assert name.startswith(row), name
             assert ("splitk" in name) == (split > 1), name
             assert np.array_equal(host(c), ref), (name, ksteps, split)
+
+
+@pytest.mark.parametrize("fam,row", [("f8_block_ref", "128x128_w2x2_k2"), ("bf16_kn", "128x128_w2x2_k2"), ("bf16_kn", "64x128_w1x4_k2")])
+def test_every_number_of_k_steps_k_major(fam, row):
+    """The same with the operands stored K-major and read as stored (transposing LDS reads in the computing waves,
+    the copying waves walking rows of k): the reference's fp8 layout with block scales, and B of a plain GEMM
+    stored K x N."""
+    M, N = 192, 320                                          # fp8_mm takes multiples of 32, as the reference does
+    Q.set_option("kmajor", 2)                                # as stored, whatever the estimate says
+    for ksteps in range(1, 14):
+        K = ksteps * (64 if fam == "bf16_kn" else 128)
+        say("k groups, K-major", row, fam, (M, N, K))
+        Q.set_option("force_config", ROWS[row])
+        Q.set_option("force_split", 1)
+        rng = np.random.default_rng(7000 + ksteps)
+        a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+        b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+        c = torch.full((M, N), -7.0, dtype=torch.float32, device="cuda")
+        if fam == "bf16_kn":
+            Q.gemm(dev(a).bfloat16(), dev(np.ascontiguousarray(b.T)).bfloat16(), c, "kn")
+            ref = R.gemm_f32acc(a, b)
+            suffix = "_nn"
+        else:
+            as_ = (2.0 ** rng.integers(-3, 4, size=(M, ksteps))).astype(np.float32)
+            bs = (2.0 ** rng.integers(-3, 4, size=((N + 127) // 128, ksteps))).astype(np.float32)
+            Q.fp8_mm(fp8_tensor(np.ascontiguousarray(R.encode_fp8(a).T)).t(), fp8_tensor(np.ascontiguousarray(R.encode_fp8(b).T)).t(),
+                     dev(np.ascontiguousarray(as_.T)).t(), dev(np.ascontiguousarray(bs.T)).t(), c)
+            ref = R.gemm_fp8_block(a, b, as_, bs)
+            suffix = "_tn"
+        name = Q.last_config()
+        assert name == row + suffix, name
+        assert np.array_equal(host(c), ref), (name, ksteps)
