@@ -63,6 +63,7 @@ struct Context {
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes; 2: never
+                                // where a K-major kernel fits the shape (for measurements and tests)
     std::string last_config;
 };
 
