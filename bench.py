@@ -453,6 +453,27 @@ def main():
         extra["cfg4_reference_layout_fp8_mm"] = gemm_entry(
             tx(lambda: Q.fp8_mm(a4r.t(), b4r.t(), as4r.t(), bs4r.t(), c4r)), f4, PEAK_TFLOPS["f8"])
         del a4r, b4r, c4r
+        # mid-size shapes with no more 128 x 128 tiles than CUs (the rows with two K groups per workgroup), microseconds
+        # per launch of a replayed graph: fp8 per-matrix, bf16, and fp8 with block scales in the reference's own storage
+        # (read as stored)
+        mm, nm_, km = 2048, 2048, 8192
+        am, sam = _quant_fp8(torch.randn(mm, km, device=dev)); bm_, sbm = _quant_fp8(torch.randn(nm_, km, device=dev))
+        cm = torch.empty(mm, nm_, dtype=torch.bfloat16, device=dev)
+        us = _graph_time([lambda: Q.scaled_gemm(am, bm_, sam, sbm, cm, mm, nm_, km, Q.SCALE_PER_MATRIX)] * 8)
+        extra["mid_fp8_2048x2048x8192"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * km / us / 1e6,
+                                           "frac_of_peak": 2.0 * mm * nm_ * km / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
+        ab16, bb16 = torch.randn(mm, km, device=dev).bfloat16(), torch.randn(nm_, km, device=dev).bfloat16()
+        us = _graph_time([lambda: Q.bf16_mm(ab16, bb16, cm)] * 8)
+        extra["mid_bf16_2048x2048x8192"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * km / us / 1e6,
+                                            "frac_of_peak": 2.0 * mm * nm_ * km / us / 1e6 / PEAK_TFLOPS["bf16"], "kernel": Q.last_config()}
+        del ab16, bb16
+        kr = 2048
+        amr, _ = _quant_fp8(torch.randn(kr, mm, device=dev)); bmr, _ = _quant_fp8(torch.randn(kr, nm_, device=dev))
+        asr = torch.rand(kr // 128, mm, device=dev) * 1.5 + 0.5; bsr = torch.rand(kr // 128, nm_ // 128, device=dev) * 1.5 + 0.5
+        us = _graph_time([lambda: Q.fp8_mm(amr.t(), bmr.t(), asr.t(), bsr.t(), cm)] * 8)
+        extra["mid_fp8_mm_reference_layout_2048"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * kr / us / 1e6,
+                                                     "frac_of_peak": 2.0 * mm * nm_ * kr / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
+        del am, bm_, cm, amr, bmr
         # transpose utility (HBM-bound: 2 * M * N * element bytes)
         for (mt, nt, dtt, nm) in ((8192, 8192, torch.bfloat16, "2B"), (7168, 6144, torch.uint8, "1B")):
             xt = torch.randint(0, 100, (mt, nt), device=dev).to(dtt)
