@@ -453,6 +453,20 @@ def main():
         extra["cfg4_reference_layout_fp8_mm"] = gemm_entry(
             tx(lambda: Q.fp8_mm(a4r.t(), b4r.t(), as4r.t(), bs4r.t(), c4r)), f4, PEAK_TFLOPS["f8"])
         del a4r, b4r, c4r
+        # decode-size rows against large weights streamed out of HBM (B rotates through more buffers than the memory-side
+        # cache holds): HBM-bound, bytes = B + A + C
+        for (ms_, ns_, ks_) in ((16, 28672, 8192), (128, 28672, 4096)):
+            nb_ = int(700e6 // (ns_ * ks_)) + 1
+            bs_ = [_quant_fp8(torch.randn(ns_, ks_, device=dev))[0] for _ in range(nb_)]
+            as_, sas_ = _quant_fp8(torch.randn(ms_, ks_, device=dev))
+            one_ = torch.ones(1, device=dev)
+            cs_ = torch.empty(ms_, ns_, dtype=torch.bfloat16, device=dev)
+            us = _graph_time([(lambda bq=bq: Q.scaled_gemm(as_, bq, sas_, one_, cs_, ms_, ns_, ks_, Q.SCALE_PER_MATRIX)) for bq in bs_])
+            nbytes = ns_ * ks_ + ms_ * ks_ + ms_ * ns_ * 2
+            extra["stream_fp8_%dx%dx%d" % (ms_, ns_, ks_)] = {
+                "us_per_launch": us, "GBps": nbytes / us / 1e3, "frac_of_hbm_peak": nbytes / us / 1e3 / PEAK_HBM_GBS,
+                "buffers": nb_, "algorithmic_bytes": nbytes, "kernel": Q.last_config()}
+            del bs_
         # mid-size shapes with no more 128 x 128 tiles than CUs (the rows with two K groups per workgroup), microseconds
         # per launch of a replayed graph: fp8 per-matrix, bf16, and fp8 with block scales in the reference's own storage
         # (read as stored)

@@ -66,6 +66,7 @@ struct GemmArgs {
     int out_dtype;        // qgemm_dtype_t of C
     int per_matrix_scale; // multiply by as[0]*bs[0] in the epilogue
     int vec_store;        // 0: scalar stores; 1: C and ldc allow 4-element vector stores; 2: also 16-byte row pieces
+    uint32_t k_rot;                  // simple pipeline and skinny-M kernel: workgroup i starts its K loop (i * k_rot) % nk steps in (0: at 0)
     uint32_t stagger, stagger_wgs;   // the first stagger_wgs workgroups start (id / 8 % 4) * stagger microseconds late (0: off)
     unsigned long long *dbg_cycles;   // measurement builds only (QGEMM_STAMP): time stamps per wave
 };
@@ -364,7 +365,20 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const int ld_chunk_km = (lane & 7) ^ kmajor_swz<C::ES>(ld_r + 16 * ((wave >> 1) & 1));
     const uint32_t voff_a = ld_r * p.lda + (C::KMA ? ld_chunk_km : ld_chunk) * 16;
     const uint32_t voff_b = ld_r * p.ldb + (C::KMB ? ld_chunk_km : ld_chunk) * 16;
-    auto load_soff = [&](int i, int kt) -> uint32_t {                   // scalar: row block + K step
+    // K step the loop's step kt stands for (rotated start, simple pipeline only: the pipelined kernels run
+    // compute-bound shapes, whose workgroups share panels and should stay in step)
+    constexpr bool K_ROT = C::PIPE == PIPE_SIMPLE;
+    const int k_first = K_ROT && p.k_rot && nk > 0 ? (int)((wg * p.k_rot) % (uint32_t)nk) : 0;
+    auto kpos = [&](int kt) -> int {
+        if constexpr (K_ROT) {
+            const int k = kt + k_first;
+            return k >= nk ? k - nk : k;
+        } else {
+            return kt;
+        }
+    };
+    auto load_soff = [&](int i, int kt_loop) -> uint32_t {              // scalar: row block + K step
+        const int kt = kpos(kt_loop);
         const bool is_a = i < LPT_A0;
         const uint32_t blk = (wave >> 1) + (is_a ? i : i - LPT_A0) * (C::NW / 2);
         const uint32_t ld = is_a ? p.lda : p.ldb;
@@ -431,7 +445,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     }
     auto fetch_scales = [&](int kt) {          // start the loads for K step kt
         if constexpr (C::BLOCK_SCALE) {
-            const uint32_t kb = kbeg + kt;
+            const uint32_t kb = kbeg + kpos(kt);
 #pragma unroll
             for (int j = 0; j < NLD; ++j)
                 as_raw[j] = __builtin_amdgcn_raw_buffer_load_b32(ras, as_voff, (64 * j * p.as_ms + kb * p.as_ks) * 4, 0);
@@ -1058,8 +1072,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // scalar offset of row block blk of an operand at K step kt: as load_soff
                 auto soff_k2 = [&](bool kmajor, uint32_t blk, uint32_t ld, int kt) -> uint32_t {
                     constexpr uint32_t BPP = C::KE / 16;                        // row blocks per panel
-                    if (kmajor) return ((uint32_t)kt * C::KE + (blk % BPP) * 16) * ld + (blk / BPP) * 128;
-                    return blk * 16 * ld + (uint32_t)kt * C::BKB;
+                    const uint32_t k = (uint32_t)kpos(kt);
+                    if (kmajor) return (k * C::KE + (blk % BPP) * 16) * ld + (blk / BPP) * 128;
+                    return blk * 16 * ld + k * C::BKB;
                 };
                 auto issue_stage_k2 = [&](int kt) {
                     char *stage = smem + (kt % NS) * C::STAGE_BYTES + pw * 1024;
@@ -1074,7 +1089,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     }
                     if constexpr (C::BLOCK_SCALE) {
                         lds_void *dst = (lds_void *)(smem + NS * C::STAGE_BYTES + (kt % NS) * 512 + (wave & 1) * 256);
-                        __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 4, as_voff_k2, (kbeg + (uint32_t)kt) * p.as_ks * 4, 0, 0);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 4, as_voff_k2, (kbeg + (uint32_t)kpos(kt)) * p.as_ks * 4, 0, 0);
                     }
                 };
 #pragma unroll
@@ -1093,7 +1108,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         const char *sc = smem + NS * C::STAGE_BYTES + (mine % NS) * 512 + (wm * C::WM + (lane & 15)) * 4;
 #pragma unroll
                         for (int a = 0; a < C::TM; ++a) as_cur[a] = *(const float *)(sc + a * 64);
-                        const uint32_t kb = kbeg + (uint32_t)mine;
+                        const uint32_t kb = kbeg + (uint32_t)kpos(mine);
 #pragma unroll
                         for (int j = 0; j < NBS; ++j)
                             bs_cur[j] = p.bs[__builtin_amdgcn_readfirstlane(bs_off[j] + kb * p.bs_ks)];

@@ -105,14 +105,23 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     const int fr = lane & 15, fg = lane >> 4;
     const int off0 = lds_slot(fr, fg) * 16, off1 = lds_slot(fr, 4 + fg) * 16;
 
+    // K step the loop's step kt stands for: the workgroup starts k_first steps in and wraps round (GemmArgs::k_rot);
+    // steps past the end stay past the end (they read zeros)
+    const int k_first = p.k_rot && nk > 0 ? (int)((wg * p.k_rot) % (uint32_t)nk) : 0;
+    auto kpos = [&](int kt) -> int {
+        const int k = kt + k_first;
+        return kt >= nk ? kt : (k >= nk ? k - nk : k);
+    };
     // copies: n kilobytes of step kt (rows 8 * first ..) of A or B into ring slots slot, slot + 1, ...
-    auto copy_a = [&](int kt, int first, int n, int slot) {
+    auto copy_a = [&](int kt_loop, int first, int n, int slot) {
+        const int kt = kpos(kt_loop);
 #pragma unroll
         for (int i = 0; i < n; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void *)(ring + (slot + i) * 1024), 16, voff_a,
                                                      (first + i) * 8 * p.lda + (uint32_t)kt * 128, 0, 0);
     };
-    auto copy_b_part = [&](int kt, int first, int n, int slot) {
+    auto copy_b_part = [&](int kt_loop, int first, int n, int slot) {
+        const int kt = kpos(kt_loop);
 #pragma unroll
         for (int i = 0; i < n; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void *)(ring + (slot + i) * 1024), 16, voff_b,
@@ -165,7 +174,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
         if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const uint32_t kb = kbeg + (uint32_t)(k + s * C::NW);
+                const uint32_t kb = kbeg + (uint32_t)kpos(k + s * C::NW);
                 // (a step past the end of K multiplies zeros: any finite scale will do, so keep the reads inside)
                 const uint32_t kbc = kb < p.ksteps ? kb : p.ksteps - 1;
 #pragma unroll
