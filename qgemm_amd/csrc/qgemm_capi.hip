@@ -313,8 +313,14 @@ int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps
 // against skinny kernel: 16 x 7168 x 2048 7.6 / 5.4, 64 x 7168 x 2048 9.0 / 6.7, 128 x 7168 x 2048 11.0 / 8.2,
 // 16 x 7168 x 8192 24.6 / 15.2, 32 x 4096 x 4096 12.7 / 8.3, 128 x 4096 x 4096 18.3 / 12.5, 16 x 1024 x 1024
 // 5.6 / 3.1; with K = 1024 and more than 16 rows or K = 512 the narrow tiles stay ahead (64 x 8192 x 1024 5.0 / 5.2,
-// 128 x 7168 x 512 4.6 / 6.0).  It never wants a K split on top: one makes it slower wherever it was tried.  The same
-// rule serves block scales (B resident: 16 x 7168 x 2048 10.8 / 6.6, 128 x 7168 x 2048 15.7 / 9.5).
+// 128 x 7168 x 512 4.6 / 6.0).  The same rule serves block scales (B resident: 16 x 7168 x 2048 10.8 / 6.6,
+// 128 x 7168 x 2048 15.7 / 9.5).
+// A K split across workgroups on top pays only where the strips leave at least half of the CUs without work and K is
+// long: a workgroup moves its strip of B and its rows of A at about 45 GB/s, a split divides that time and adds a
+// reduction launch of about 4.5 us.  B out of HBM, microseconds per launch, one workgroup per strip against the split
+// this estimate picks: 16 x 4096 x 14336 fp8 20.6 / 17.2 (two slices), bf16 37.1 / 26.9; 64 x 4096 x 14336 27.3 / 22.7,
+// bf16 53.7 / 37.2; 64 x 2048 x 8192 15.2 / 11.3 (four slices), bf16 26.8 / 14.7; no split for 16 x 4096 x 4096 (7.6
+// against 9.5 with two slices) and none where the strips fill the CUs (16 x 8192 x 8192 15.2 against 18.8).
 // kmaj: the table is a K-major family, which has no narrow tiles: the estimate then serves every M
 int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
                    bool may_split, uint32_t *nsplit_out) {
@@ -340,6 +346,18 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     for (int i = 0; i < count; ++i)
         if (tab[i].kgroups == 8 && tab[i].bn == 32 && (size_t)tab[i].bm >= M) {        // (rows of the table in ascending height)
             *nsplit_out = 1;
+            const size_t strips = (N + 31) / 32;
+            if (may_split && strips * 2 <= (size_t)cus) {
+                const double t_one = (double)(32 + tab[i].bm) * ksteps * 128.0 / 45.0e3;     // us, one workgroup per strip
+                double best = t_one;
+                for (uint32_t ns = 2; ns <= 8 && strips * ns <= (size_t)cus && ksteps / ns >= 8; ++ns) {
+                    const double t = t_one / ns + 4.5;
+                    if (t < best) {
+                        best = t;
+                        *nsplit_out = ns;
+                    }
+                }
+            }
             return i;
         }
     return vi;

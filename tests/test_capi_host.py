@@ -108,7 +108,12 @@ def test_plan_names_the_kernel_without_a_device():
     for m, name in ((16, "skinny_16x32_k8"), (64, "skinny_64x32_k8"), (128, "skinny_128x32_k8")):
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
         assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
-    assert plan(Q.DT_BF16, 0, 0, 24, 4096, 4096) == "skinny_32x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 24, 4096, 4096) == "skinny_32x32_k8"
+    # ... with a K split across workgroups on top where the strips leave half of the CUs idle and K is long
+    assert plan(Q.DT_BF16, 0, 0, 24, 4096, 4096) == "skinny_32x32_k8_splitk2"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 4096, 14336) == "skinny_16x32_k8_splitk2"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 2048, 8192) == "skinny_64x32_k8_splitk4"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 8192, 8192) == "skinny_16x32_k8"
     # ... but not with few K steps or where the estimate prefers wide tiles
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 7168, 512) == "128x32_w4x1_dma"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 8192, 1024) == "64x32_w4x1_dma"
