@@ -341,12 +341,26 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
                     return i;
                 }
     }
-    if (vi < 0 || kmaj || M > 128 || tab[vi].bn != 32 || tab[vi].kgroups != 1) return vi;
+    if (vi < 0 || kmaj || M > 128) return vi;
+    const size_t strips = (N + 31) / 32;
+    // 33 .. 64 rows against so many columns that the 32-column strips need a second round of CUs while 64-column
+    // strips fit in one: the 64 x 64 form (half the strips, each row of A fetched half as often).  B out of HBM:
+    // 64 x 14336 x 4096 bf16 34.3 -> 26.7 us, fp8 20.4 -> 17.0; 48 rows 33.4 -> 27.4 and 19.4 -> 16.5.
+    if (M > 32 && M <= 64 && ksteps >= 16 && strips > (size_t)cus && (N + 63) / 64 <= (size_t)cus)
+        for (int i = 0; i < count; ++i)
+            if (tab[i].kgroups == 8 && tab[i].bm == 64 && tab[i].bn == 64) {
+                *nsplit_out = 1;
+                return i;
+            }
+    // 65 .. 128 rows come out of the estimate above, whose times per step are those of operands that sit in the caches;
+    // with B streamed out of memory the skinny-M kernel is ahead wherever its strips fit one round of CUs and K is
+    // not long enough for a K split to pay (128 x 7168 x 2048 bf16 17.8 -> 13.6 us, 128 x 8192 x 8192 fp8 26.9 -> 24.8)
+    const bool mid_rows = M > 64 && strips <= (size_t)cus && ksteps >= 16 && ksteps <= 64;
+    if (!mid_rows && (tab[vi].bn != 32 || tab[vi].kgroups != 1)) return vi;
     if (ksteps < 8 || (ksteps < 16 && M > 16)) return vi;
     for (int i = 0; i < count; ++i)
         if (tab[i].kgroups == 8 && tab[i].bn == 32 && (size_t)tab[i].bm >= M) {        // (rows of the table in ascending height)
             *nsplit_out = 1;
-            const size_t strips = (N + 31) / 32;
             if (may_split && strips * 2 <= (size_t)cus) {
                 const double t_one = (double)(32 + tab[i].bm) * ksteps * 128.0 / 45.0e3;     // us, one workgroup per strip
                 double best = t_one;

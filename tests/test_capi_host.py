@@ -114,6 +114,13 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 4096, 14336) == "skinny_16x32_k8_splitk2"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 2048, 8192) == "skinny_64x32_k8_splitk4"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 8192, 8192) == "skinny_16x32_k8"
+    # 33 .. 64 rows whose 32-column strips need a second round of CUs: 64-column strips; 65 .. 128 rows whose strips
+    # fit one round and K is not long: the skinny-M kernel rather than what the estimate (of resident operands) likes
+    assert plan(Q.DT_BF16, 0, 0, 64, 14336, 4096) == "skinny_64x64_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 8192, 8192) == "skinny_64x32_k8"
+    assert plan(Q.DT_BF16, 0, 0, 128, 7168, 2048) == "skinny_128x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 8192, 8192) == "skinny_128x32_k8"
+    assert plan(Q.DT_BF16, 0, 0, 128, 8192, 8192) == "128x128_w2x2_k2_splitk4"
     # ... but not with few K steps or where the estimate prefers wide tiles
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 7168, 512) == "128x32_w4x1_dma"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 8192, 1024) == "64x32_w4x1_dma"
