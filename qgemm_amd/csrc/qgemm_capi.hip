@@ -356,7 +356,11 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     // with B streamed out of memory the skinny-M kernel is ahead wherever its strips fit one round of CUs and K is
     // not long enough for a K split to pay (128 x 7168 x 2048 bf16 17.8 -> 13.6 us, 128 x 8192 x 8192 fp8 26.9 -> 24.8)
     const bool mid_rows = M > 64 && strips <= (size_t)cus && ksteps >= 16 && ksteps <= 64;
-    if (!mid_rows && (tab[vi].bn != 32 || tab[vi].kgroups != 1)) return vi;
+    // (up to 64 rows the choice above takes a wide tile with a K split where 32-column tiles of its height would need
+    // more than two rounds; up to two rounds of strips the skinny-M kernel is ahead of that too: 32 x 14336 x 4096 fp8
+    // 24.6 -> 17.2 us, bf16 36.4 -> 29.7; with 896 strips the wide tiles stay, 32 x 28672 x 8192 46.8 against 55.1)
+    const bool few_strips = M <= 64 && strips <= 2 * (size_t)cus && ksteps >= 16;
+    if (!mid_rows && !few_strips && (tab[vi].bn != 32 || tab[vi].kgroups != 1)) return vi;
     if (ksteps < 8 || (ksteps < 16 && M > 16)) return vi;
     for (int i = 0; i < count; ++i)
         if (tab[i].kgroups == 8 && tab[i].bn == 32 && (size_t)tab[i].bm >= M) {        // (rows of the table in ascending height)
