@@ -221,6 +221,48 @@ def one_shape(Q, torch, dev, spec, launches):
             "tflops": round(2.0 * M * N * K / us / 1e6, 1)}
 
 
+STREAM_SHAPES = [(1, 8192, 8192), (16, 4096, 4096), (16, 4096, 14336), (64, 4096, 14336), (16, 8192, 8192), (64, 8192, 8192),
+                 (128, 8192, 8192), (16, 14336, 4096), (32, 14336, 4096), (64, 14336, 4096), (128, 14336, 4096),
+                 (16, 28672, 8192), (64, 28672, 8192), (128, 28672, 4096), (32, 8192, 28672), (16, 7168, 2048),
+                 (64, 7168, 2048), (128, 7168, 2048)]
+
+
+def stream_sweep(Q, torch, dev):
+    """Decode-size row counts against weight matrices streamed out of HBM: B rotates through enough buffers (700 MB) that
+    no launch finds its B in the 256 MB memory-side cache; this library and the vendor library, each as a replayed graph
+    of one launch per buffer.  Microseconds per launch and TB/s of algorithmic bytes (B + A + C)."""
+    rows = []
+    for fam in ("fp8", "bf16"):
+        for (M, N, K) in STREAM_SHAPES:
+            es = 1 if fam == "fp8" else 2
+            nbuf = max(2, int(700e6 // (N * K * es)) + 1)
+            c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            if fam == "fp8":
+                bs = [_quant_fp8(torch.randn(N, K, device=dev))[0] for _ in range(nbuf)]
+                a, sa = _quant_fp8(torch.randn(M, K, device=dev))
+                sb = torch.ones(1, device=dev)
+                ours = [(lambda b=b: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)) for b in bs]
+                theirs = [(lambda b=b: torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)) for b in bs]
+            else:
+                bs = [torch.randn(N, K, device=dev).bfloat16() for _ in range(nbuf)]
+                a = torch.randn(M, K, device=dev).bfloat16()
+                ours = [(lambda b=b: Q.bf16_mm(a, b, c)) for b in bs]
+                theirs = [(lambda b=b: torch.matmul(a, b.t(), out=c)) for b in bs]
+            nbytes = (N * K + M * K) * es + M * N * 2
+            row = {"type": fam, "M": M, "N": N, "K": K, "buffers": nbuf}
+            t_ours = _graph_time(ours, reps=6)
+            row.update({"this_library_us": round(t_ours, 1), "this_library_TBps": round(nbytes / t_ours / 1e6, 2), "kernel": Q.last_config()})
+            try:
+                t_theirs = _graph_time(theirs, reps=6)
+                row.update({"vendor_us": round(t_theirs, 1), "vendor_TBps": round(nbytes / t_theirs / 1e6, 2), "ratio": round(t_ours / t_theirs, 3)})
+            except Exception as e:                  # a vendor row that does not run is reported, not hidden
+                row["error"] = str(e)[:200]
+            rows.append(row)
+            print("[stream]", json.dumps(row), file=sys.stderr, flush=True)
+            del bs
+    return rows
+
+
 def skinny_probe(Q, torch, dev):
     """Where a launch of the skinny-M kernel spends its time (config 5 shapes, fp8):
       * graph-replay time per launch with B resident against the number of 32-column strips (= workgroups), K and
@@ -288,6 +330,9 @@ def main():
     ap.add_argument("--vendor-sweep", action="store_true",
                     help="only time this library against the vendor library (torch.matmul, torch._scaled_mm, "
                          "torch._int_mm) over a list of shapes, interleaved, print one JSON line and exit")
+    ap.add_argument("--stream-sweep", action="store_true",
+                    help="only time decode-size shapes whose weights are streamed out of HBM, this library and the vendor "
+                         "library from replayed graphs, print one JSON line and exit")
     ap.add_argument("--shape", default="",
                     help="only run this library on one shape, e.g. fp8:2048x2048x8192 (fp8 | fp8block | int8 | bf16 | fp16), "
                          "--steps launches from a replayed graph; print one JSON line and exit")
@@ -316,6 +361,9 @@ def main():
     dev = "cuda:0"
     if args.shape:
         print(json.dumps({"shape": one_shape(Q, torch, dev, args.shape, max(1, min(args.steps, 200)))}))
+        return 0
+    if args.stream_sweep:
+        print(json.dumps({"stream_sweep": stream_sweep(Q, torch, dev)}))
         return 0
     if args.vendor_sweep:
         print(json.dumps({"vendor_sweep": vendor_sweep(Q, torch, dev)}))
