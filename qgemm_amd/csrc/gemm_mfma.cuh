@@ -66,7 +66,7 @@ struct GemmArgs {
     int out_dtype;        // qgemm_dtype_t of C
     int per_matrix_scale; // multiply by as[0]*bs[0] in the epilogue
     int vec_store;        // 0: scalar stores; 1: C and ldc allow 4-element vector stores; 2: also 16-byte row pieces
-    uint32_t k_rot;                  // simple pipeline and skinny-M kernel: workgroup i starts its K loop (i * k_rot) % nk steps in (0: at 0)
+    uint32_t k_rot;                  // simple pipeline and skinny-M kernel: the workgroups of column tile i start their K loops (i * k_rot) % nk steps in (0: at 0)
     uint32_t stagger, stagger_wgs;   // the first stagger_wgs workgroups start (id / 8 % 4) * stagger microseconds late (0: off)
     unsigned long long *dbg_cycles;   // measurement builds only (QGEMM_STAMP): time stamps per wave
 };
@@ -368,7 +368,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // K step the loop's step kt stands for (rotated start, simple pipeline only: the pipelined kernels run
     // compute-bound shapes, whose workgroups share panels and should stay in step)
     constexpr bool K_ROT = C::PIPE == PIPE_SIMPLE;
-    const int k_first = K_ROT && p.k_rot && nk > 0 ? (int)((wg * p.k_rot) % (uint32_t)nk) : 0;
+    const int k_first = K_ROT && p.k_rot && nk > 0 ? (int)((tn * p.k_rot) % (uint32_t)nk) : 0;    // by column tile: the row tiles of a panel of B stay in step
     auto kpos = [&](int kt) -> int {
         if constexpr (K_ROT) {
             const int k = kt + k_first;

@@ -105,9 +105,10 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     const int fr = lane & 15, fg = lane >> 4;
     const int off0 = lds_slot(fr, fg) * 16, off1 = lds_slot(fr, 4 + fg) * 16;
 
-    // K step the loop's step kt stands for: the workgroup starts k_first steps in and wraps round (GemmArgs::k_rot);
+    // K step the loop's step kt stands for: the workgroups of a column strip start k_first steps in and wrap round
+    // (GemmArgs::k_rot);
     // steps past the end stay past the end (they read zeros)
-    const int k_first = p.k_rot && nk > 0 ? (int)((wg * p.k_rot) % (uint32_t)nk) : 0;
+    const int k_first = p.k_rot && nk > 0 ? (int)((tn * p.k_rot) % (uint32_t)nk) : 0;
     auto kpos = [&](int kt) -> int {
         const int k = kt + k_first;
         return kt >= nk ? kt : (k >= nk ? k - nk : k);

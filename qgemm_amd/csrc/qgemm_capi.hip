@@ -60,7 +60,7 @@ struct Context {
 #if QGEMM_DEBUG_BUILD
     long dbg_ptr = 0;           // measurement builds: device buffer for the kernels' time stamps (GemmArgs::dbg_cycles)
 #endif
-    long k_rot = -1;            // -1: rotated K start for at most 128 rows (see plan_nt), 0: never, n: steps per workgroup
+    long k_rot = -1;            // -1: rotated K start for at most 256 rows (see plan_nt), 0: never, n: steps per column tile
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes; 2: never
@@ -545,12 +545,13 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
     a.tiles_m = (uint32_t)((q.M + v.bm - 1) / v.bm);
     a.tiles_n = (uint32_t)((q.N + v.bn - 1) / v.bn);
     a.group_m = g_ctx.force_group_m > 0 ? (uint32_t)g_ctx.force_group_m : 8;
-    // Few rows (every workgroup streams a strip of B of its own out of memory, all of them at the same k): workgroup i
-    // starts its K loop k_rot * i steps in and wraps round, so that at any time the workgroups read at different offsets
+    // Few rows (every workgroup streams a strip of B of its own out of memory, all of them at the same k): the workgroups
+    // of column tile i (which share that strip of B and stay in step) start their K loops k_rot * i steps in and wrap
+    // round, so that at any time the column tiles read at different offsets
     // inside their rows; with rows a power of two apart they otherwise all ask the same few memory channels
     // (16 x 28672 x 8192 fp8 with B out of HBM: 53 us from step 0, 45 - 46 us with 1, 2, 3 or 16 steps per workgroup,
     // 53 again with 32, i.e. 4 KiB; 8 steps are worse than none for the skinny-M kernel, whose waves share 16 steps).
-    a.k_rot = g_ctx.k_rot >= 0 ? (uint32_t)g_ctx.k_rot : (q.M <= 128 ? 3u : 0u);
+    a.k_rot = g_ctx.k_rot >= 0 ? (uint32_t)g_ctx.k_rot : (q.M <= 256 ? 3u : 0u);
     a.as_ms = q.as_ms;
     a.as_ks = q.as_ks;
     a.bs_ns = q.bs_ns;
