@@ -63,6 +63,8 @@ struct GemmArgs {
     uint64_t split_stride;
     uint32_t as_ms, as_ks, bs_ns, bs_ks;
     uint32_t nb_max;      // ceil(N/128) - 1
+    uint32_t as_groups;   // rows with two K groups, block scales: a_scale is K-contiguous (as_ks == 1), 16-byte aligned rows,
+                          // every K slice and k_rot a multiple of four steps: the scales travel four K blocks at a time
     int out_dtype;        // qgemm_dtype_t of C
     int per_matrix_scale; // multiply by as[0]*bs[0] in the epilogue
     int vec_store;        // 0: scalar stores; 1: C and ldc allow 4-element vector stores; 2: also 16-byte row pieces
@@ -159,7 +161,8 @@ struct GemmCfg {
     // Block scales with K groups: the a_scale values of a stage (one float per tile row, at most 128) travel to LDS
     // like the operands, 512 bytes per stage behind the ring, so that every copy of the loop is of one kind and the
     // wave's own count of copies in flight stays exact (a register load among them makes the compiler wait for all).
-    static constexpr int SCALE_LDS = (BLOCK_SCALE_ && KGROUPS_ == 2) ? NSTAGE * 512 : 0;
+    // (or, K-contiguous a_scale: four slots of BM rows x four K blocks, see the K loop)
+    static constexpr int SCALE_LDS = (BLOCK_SCALE_ && KGROUPS_ == 2) ? (NSTAGE * 512 > 64 * BM_ ? NSTAGE * 512 : 64 * BM_) : 0;
     static constexpr int LDS_BYTES = (A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES) + SCALE_LDS;
     static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && (!BLOCK_SCALE || KGROUPS_ == 2) &&
                                    (KMAJ_ == 0 || KGROUPS_ == 2) && STAGES_ >= 2 && STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
@@ -1060,6 +1063,14 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // Block scales: each copying wave adds one 4-byte-per-lane copy per stage that brings the a_scale values
             // of 64 tile rows (even waves rows 0 - 63, odd waves rows 64 - 127: the same bytes to the same place from
             // two waves, so that all of them count alike) to the stage's 512 bytes behind the ring.
+            // That is one request per row and stage, as many again as the operands' own when the caller's a_scale is
+            // K-contiguous (every lane another cache line: 2048 x 2048 x 8192 took 46 us where the same copies at
+            // contiguous addresses take 37).  Where the host finds such an a_scale aligned for it (GemmArgs::as_groups)
+            // a lane fetches the scales of four K blocks of its row at once, 16 bytes, in front of every fourth stage
+            // (waves 0 and 1 of the copying four, 64 rows each), into slot (kt / 4) % 4 of four behind the ring:
+            // [row][4 K blocks].  Slot i is refilled for stage 4 i + 16, issued in phase 4 i + 17 - NS, after the last
+            // read of stage 4 i + 3.  These copies are not counted: a wave that waits until (NS - 2) * NPC copies are
+            // left in flight has then waited for one or two operand copies more than it had to.
             constexpr int NPC = C::NLOAD / C::NPROD;                        // operand copies per stage and copying wave
             constexpr int CPS = NPC + (C::BLOCK_SCALE ? 1 : 0);
             static_assert(C::NPROD == 4 && C::NLOAD % 4 == 0 && C::RBA % 2 == 0 && (NS - 2) * CPS <= 63,
@@ -1088,26 +1099,47 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                             __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 0);
                     }
                     if constexpr (C::BLOCK_SCALE) {
-                        lds_void *dst = (lds_void *)(smem + NS * C::STAGE_BYTES + (kt % NS) * 512 + (wave & 1) * 256);
-                        __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 4, as_voff_k2, (kbeg + (uint32_t)kpos(kt)) * p.as_ks * 4, 0, 0);
+                        if (!p.as_groups) {
+                            lds_void *dst = (lds_void *)(smem + NS * C::STAGE_BYTES + (kt % NS) * 512 + (wave & 1) * 256);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 4, as_voff_k2, (kbeg + (uint32_t)kpos(kt)) * p.as_ks * 4, 0, 0);
+                        }
+                    }
+                };
+                auto issue_scale_group = [&](int kt) {          // in front of the copies of stage kt
+                    if constexpr (C::BLOCK_SCALE) {
+                        if (p.as_groups && (kt & 3) == 0 && pw < C::BM / 64) {
+                            lds_void *dst = (lds_void *)(smem + NS * C::STAGE_BYTES + ((kt >> 2) & 3) * (16 * C::BM) + pw * 1024);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 16, as_voff_k2, (kbeg + (uint32_t)kpos(kt)) * 4, 0, 0);
+                        }
                     }
                 };
 #pragma unroll
                 for (int j = 0; j < NS - 1; ++j)
-                    if (j < nk) issue_stage_k2(j);
+                    if (j < nk) {
+                        issue_scale_group(j);
+                        issue_stage_k2(j);
+                    }
+                const bool counted = !C::BLOCK_SCALE || !p.as_groups;       // the scale copies are among the CPS of a stage
                 for (int ph = 0; ph <= nk; ++ph) {
-                    if (ph + NS - 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * CPS));
-                    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
+                    if (ph + NS - 2 >= nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
+                    else if (counted) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * CPS));
+                    else __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * NPC));
                     phase_barrier();
-                    if (ph + NS - 1 < nk) issue_stage_k2(ph + NS - 1);
+                    if (ph + NS - 1 < nk) {
+                        issue_scale_group(ph + NS - 1);
+                        issue_stage_k2(ph + NS - 1);
+                    }
                 }
             } else {
                 v4i fa[C::TM][2], fb[C::TN][2];
                 auto read_stage = [&](int mine) {
                     if constexpr (C::BLOCK_SCALE) {
-                        const char *sc = smem + NS * C::STAGE_BYTES + (mine % NS) * 512 + (wm * C::WM + (lane & 15)) * 4;
+                        const int tr = wm * C::WM + (lane & 15);                    // tile row of this lane in row block 0
+                        const char *sc = smem + NS * C::STAGE_BYTES +
+                                         (p.as_groups ? ((mine >> 2) & 3) * (16 * C::BM) + tr * 16 + (mine & 3) * 4 : (mine % NS) * 512 + tr * 4);
+                        const int rb = p.as_groups ? 256 : 64;                      // bytes from one row block to the next
 #pragma unroll
-                        for (int a = 0; a < C::TM; ++a) as_cur[a] = *(const float *)(sc + a * 64);
+                        for (int a = 0; a < C::TM; ++a) as_cur[a] = *(const float *)(sc + a * rb);
                         const uint32_t kb = kbeg + (uint32_t)kpos(mine);
 #pragma unroll
                         for (int j = 0; j < NBS; ++j)
@@ -1130,27 +1162,28 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     if constexpr (C::BLOCK_SCALE) {
                         // P * (as * bs), then accumulate (hip_mix_gemm_kernel.cpp:241 has (P * as) * bs: the factor
                         // formed first is one multiply per row and K block instead of four per MFMA).  Each MFMA starts
-                        // from zero; its partial product is folded into the running sum one MFMA later, so that the
-                        // four FMAs of a tile run under the MFMA of the next (straight after its own MFMA they would
-                        // wait for it, and the next MFMA for them: 60 cycles a tile instead of 32).
-                        constexpr int NT = C::TM * C::TN;
+                        // from zero; its partial product is folded into the running sum two MFMAs later, so that the
+                        // four FMAs of a tile run under the MFMAs that follow (straight after its own MFMA they would
+                        // wait for it, and the next MFMA for them: 60 cycles a tile instead of 32; one MFMA behind, a
+                        // register-only loop of this pattern takes 35 cycles a tile, two behind 33).
+                        constexpr int NT = C::TM * C::TN, BEHIND = 2;
                         float f[C::TM][NBS];
 #pragma unroll
                         for (int a = 0; a < C::TM; ++a)
 #pragma unroll
                             for (int j = 0; j < NBS; ++j) f[a][j] = as_cur[a] * bs_cur[j];
-                        v4f part[2];
+                        v4f part[BEHIND + 1];
 #pragma unroll
-                        for (int i = 0; i <= NT; ++i) {
+                        for (int i = 0; i < NT + BEHIND; ++i) {
                             if (i < NT) {
                                 const int a = i % C::TM, b = i / C::TM;
-                                part[i & 1] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                                part[i % (BEHIND + 1)] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
                             }
-                            __builtin_amdgcn_sched_barrier(0);       // MFMA i first, the FMAs of tile i-1 under it
-                            if (i > 0) {
-                                const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
+                            __builtin_amdgcn_sched_barrier(0);       // MFMA i first, the FMAs of tile i-2 under it
+                            if (i >= BEHIND) {
+                                const int t = i - BEHIND, pa = t % C::TM, pb = t / C::TM;
 #pragma unroll
-                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f[pa][(pb * 16) / 128];
+                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[t % (BEHIND + 1)][r] * f[pa][(pb * 16) / 128];
                             }
                             __builtin_amdgcn_sched_barrier(0);
                         }

@@ -60,6 +60,7 @@ struct Context {
 #if QGEMM_DEBUG_BUILD
     long dbg_ptr = 0;           // measurement builds: device buffer for the kernels' time stamps (GemmArgs::dbg_cycles)
 #endif
+    long as_groups = 1;         // 0: a_scale always one K block per copy on the rows with two K groups (see run_nt)
     long k_rot = -1;            // -1: rotated K start for at most 256 rows (see plan_nt), 0: never, n: steps per column tile
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
@@ -267,10 +268,11 @@ struct TileModel {
 };
 // (block scales, graph replays: 256 x 256 2048 x 4608 x 7168 77 us, 1536 x 7168 x 2048 27.6; 128 x 128 1024 x 7168 x 2048 25.9,
 // 1024 x 4608 x 7168 75.0; 64 x 128 1024 x 4608 x 7168 69.9, 512 x 4608 x 7168 47.8; K groups 128 x 128 2048 x 2048 x 2048 /
-// 8192 14 / 43, 64 x 128 512 x 4096 x 4096 18; 128 x 32 256 x 7168 x 2048 12.9)
+// 8192 14 / 43, 64 x 128 512 x 4096 x 4096 18, and with the a_scale values of four K blocks per copy (GemmArgs::as_groups)
+// 38 - 41 and 15.3; 128 x 32 256 x 7168 x 2048 12.9)
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.32, 1.04},
-                                 {128, 128, 1, 0.43, 0.43, 4.5, true, 1, 0.55, 0.55},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
-                                 {64, 128, 1, 0.27, 0.27, 4.5, true, 1, 0.40, 0.40},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
+                                 {128, 128, 1, 0.43, 0.43, 4.5, true, 1, 0.50, 0.50},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
+                                 {64, 128, 1, 0.27, 0.27, 4.5, true, 1, 0.34, 0.34},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60}};
 // rows with two K groups: two sets of computing waves on a tile that otherwise has one (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 
@@ -609,6 +611,15 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
     a.as_ks = q.as_ks;
     a.bs_ns = q.bs_ns;
     a.bs_ks = q.bs_ks;
+    a.as_groups = 0;
+    if (q.block && v.kgroups == 2 && g_ctx.as_groups) {
+        // K-contiguous a_scale on the rows with two K groups: four K blocks of a row per copy (GemmArgs::as_groups) where
+        // rows and K slices start at multiples of four blocks; the rotated start then moves by four steps a column tile
+        const bool slices4 = a.ksteps % 4 == 0 && (a.nsplit == 1 || a.ksteps_per_split % 4 == 0);
+        const bool rows16 = q.as_ks == 1 && q.as_ms % 4 == 0 && ((uintptr_t)q.as & 15u) == 0;
+        if (slices4 && rows16 && g_ctx.k_rot < 0 && a.k_rot) a.k_rot = 4;
+        a.as_groups = slices4 && rows16 && a.k_rot % 4 == 0;
+    }
 #if QGEMM_DEBUG_BUILD
     a.dbg_cycles = (unsigned long long *)g_ctx.dbg_ptr;
 #endif
@@ -908,6 +919,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
     else if (!std::strcmp(key, "stagger")) g_ctx.stagger = value;
     else if (!std::strcmp(key, "k_rot")) g_ctx.k_rot = value;
+    else if (!std::strcmp(key, "as_groups")) g_ctx.as_groups = value;
 #if QGEMM_DEBUG_BUILD
     else if (!std::strcmp(key, "dbg_ptr")) g_ctx.dbg_ptr = value;
 #endif

@@ -138,9 +138,9 @@ def test_plan_names_the_kernel_without_a_device():
     # a partly empty last round of 256 x 256 tiles: its rows become a second launch with smaller tiles
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 6144, 6144) == "256x256_w2x2_solo+128x128_w2x2_dma"
     # (block scales as this layout passes them: the twin for the first launch, the simple pipeline takes any strides;
-    # with block scales the small tiles cost more, and 6144^3 stays one launch)
+    # 6144^3: 222 us in two launches against 231 in one)
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 2560, 7680, 2048) == "256x256_w2x4_solo8_ks+128x128_w2x2_k2"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 6144, 6144) == "256x256_w2x4_solo8_ks"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 6144, 6144) == "256x256_w2x4_solo8_ks+128x128_w2x2_k2"
     # ... also when a single launch would take smaller tiles for everything, and with a rest of at most 128 rows
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 5000, 4096, 7168) == "256x256_w2x2_solo+128x128_w2x2_k2"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 7000, 7168, 2048) == "256x256_w2x2_solo+skinny_128x32_k8"

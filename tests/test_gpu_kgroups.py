@@ -18,7 +18,7 @@ ROWS = {"128x128_w2x2_k2": 16, "64x128_w1x4_k2": 17}       # rows of the variant
 @pytest.fixture(autouse=True)
 def _reset_options():
     yield
-    for k, v in (("force_config", -1), ("force_split", 0), ("kmajor", 1)):
+    for k, v in (("force_config", -1), ("force_split", 0), ("kmajor", 1), ("k_rot", -1), ("as_groups", 1)):
         Q.set_option(k, v)
 
 
@@ -91,3 +91,34 @@ def test_every_number_of_k_steps_k_major(fam, row):
         name = Q.last_config()
         assert name == row + suffix, name
         assert np.array_equal(host(c), ref), (name, ksteps)
+
+
+@pytest.mark.parametrize("row", sorted(ROWS))
+def test_block_scales_four_k_blocks_a_copy(row):
+    """K-contiguous a_scale, rows and K slices at multiples of four blocks: the copying waves bring four K blocks of a
+    row at once into one of four slots.  More than four groups (the slots are reused), a K split whose slices are
+    (8) and are not (6, 10) multiples of four, the rotated start by four steps, by three (the single-block copies take
+    over) and none, an a_scale whose rows are not 16-byte aligned (the same), and the option that switches it off:
+    every result equals the oracle bit for bit."""
+    M, N = 200, 328
+    for ksteps in (4, 8, 12, 16, 20, 40):
+        for split, k_rot, groups, shift in ((1, -1, 1, 0), (1, 0, 1, 0), (1, 4, 1, 0), (1, 8, 1, 0), (1, 3, 1, 0),
+                                            (2, -1, 1, 0), (1, -1, 0, 0), (1, -1, 1, 1), (2, 4, 1, 1)):
+            K = ksteps * 128
+            say("k groups, a_scale in groups", row, (M, N, K), "split", split, "k_rot", k_rot, "groups", groups, "shift", shift)
+            Q.set_option("force_config", ROWS[row])
+            Q.set_option("force_split", split)
+            Q.set_option("k_rot", k_rot)
+            Q.set_option("as_groups", groups)
+            rng = np.random.default_rng(31 * ksteps + split + 7 * shift)
+            a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+            b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+            as_ = (2.0 ** rng.integers(-3, 4, size=(M, ksteps))).astype(np.float32)
+            bs = (2.0 ** rng.integers(-3, 4, size=((N + 127) // 128, ksteps))).astype(np.float32)
+            as_dev = torch.empty(M * ksteps + 4, dtype=torch.float32, device="cuda")[shift:shift + M * ksteps]
+            as_dev.copy_(dev(as_).reshape(-1))
+            c = torch.full((M, N), -7.0, dtype=torch.float32, device="cuda")
+            Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), as_dev, dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
+            name = Q.last_config()
+            assert name.startswith(row) and ("splitk" in name) == (split > 1), name
+            assert np.array_equal(host(c), R.gemm_fp8_block(a, b, as_, bs)), (name, ksteps, split, k_rot, groups, shift)
