@@ -524,6 +524,10 @@ def main():
         us = _graph_time([lambda: Q.scaled_gemm(am, bm_, sam, sbm, cm, mm, nm_, km, Q.SCALE_PER_MATRIX)] * 8)
         extra["mid_fp8_2048x2048x8192"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * km / us / 1e6,
                                            "frac_of_peak": 2.0 * mm * nm_ * km / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
+        asm_ = (torch.rand(mm, km // 128, device=dev) + 0.5) / 448; bsm_ = (torch.rand(nm_ // 128, km // 128, device=dev) + 0.5) / 448
+        us = _graph_time([lambda: Q.scaled_gemm(am, bm_, asm_, bsm_, cm, mm, nm_, km, Q.SCALE_BLOCK128)] * 8)
+        extra["mid_fp8_block_2048x2048x8192"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * km / us / 1e6,
+                                                 "frac_of_peak": 2.0 * mm * nm_ * km / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
         ab16, bb16 = torch.randn(mm, km, device=dev).bfloat16(), torch.randn(nm_, km, device=dev).bfloat16()
         us = _graph_time([lambda: Q.bf16_mm(ab16, bb16, cm)] * 8)
         extra["mid_bf16_2048x2048x8192"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * km / us / 1e6,
