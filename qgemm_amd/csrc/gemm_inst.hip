@@ -138,6 +138,16 @@ static const Variant kTable[] = {
 #else
     skinny_row<4, 4>("skinny_64x64_k8"),
 #endif
+    // 256 x 128 on the solo schedule with four computing waves (128 x 64 wave tiles, one per SIMD) and four copying
+    // waves (GemmCfg::COPYW): block scales and K-major operands on a large tile, and its twin for K-contiguous a_scale
+    row_of<true, GemmCfg<INST_ARITH, (bool)INST_BLOCK, 256, 128, 2, 2, LOAD_DMA, PIPE_SOLO, 0, true, INST_KMAJ, 0, 1, false, true>,
+           CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("256x128_w2x2_cw", true),
+#if INST_BLOCK && !INST_KMAJ
+    row_of<true, GemmCfg<INST_ARITH, true, 256, 128, 2, 2, LOAD_DMA, PIPE_SOLO, 0, true, 0, 0, 1, true, true>,
+           CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("256x128_w2x2_cw_ks", false),
+#else
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+#endif
 };
 
 const Variant *INST_FN(int *count) {

@@ -102,8 +102,14 @@ enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1, PIPE_SOLO = 2 };
 // land within one step.
 template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int LOADER_ = LOAD_DMA,
           int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false, int KMAJ_ = 0, int STAGES_ = 0, int KGROUPS_ = 1,
-          bool ASK_ = false>
+          bool ASK_ = false, bool COPYW_ = false>
 struct GemmCfg {
+    // COPYW (solo pipeline, four computing waves with 128 x 64 wave tiles on a 256 x 128 tile): four more waves issue
+    // every copy of the K loop, at the places the schedule has them; the computing waves, one per SIMD, issue fragment
+    // reads, MFMAs and (block scales) the fold, and nothing that queues at the memory pipe.  Their accumulators are
+    // compiler-managed as in the 8-wave form, so block scales are possible, and since they have no copies in flight
+    // the tile may be K-major (the compiler's wait in front of a transposing read then waits for nothing).
+    static constexpr bool COPYW = COPYW_;
     // ASK (block scales, solo pipeline): a_scale is read with the K blocks contiguous, a_scale[m * as_ms + kb], the
     // arrangement of QGEMM_LAYOUT_K_CONTIGUOUS, instead of rows contiguous, a_scale[m + kb * as_ks].  A compile-time
     // choice: as a branch inside the K loop it cost the 8-wave kernel 758 spilled registers.
@@ -137,7 +143,7 @@ struct GemmCfg {
     static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int NW = WAVES_M * WAVES_N * KGROUPS_;
     // K groups: four more waves that only copy (waves NW .. NW+3, see the K loop)
-    static constexpr int NPROD = KGROUPS_ == 2 ? 4 : 0;
+    static constexpr int NPROD = (KGROUPS_ == 2 || COPYW_) ? 4 : 0;
     static constexpr int THREADS = (NW + NPROD) * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // wave tile
     static constexpr int TM = WM / 16, TN = WN / 16;            // 16x16 MFMA tiles per wave
@@ -178,7 +184,8 @@ struct GemmCfg {
     static_assert(PIPE != PIPE_PINGPONG || (NW == 8 && LOADER == LOAD_DMA), "ping-pong needs 8 waves and the DMA loader");
     static_assert(PIPE != PIPE_SOLO || ((NW == 4 || NW == 8) && LOADER == LOAD_DMA && A3 && TM % 4 == 0 && TM >= 8 && TN >= 4),
                   "solo: 4 or 8 waves, DMA loader, A triple-buffered, at least 8 rows of at least 4 MFMAs per step");
-    static_assert(PIPE != PIPE_SOLO || !BLOCK_SCALE || NW == 8,
+    static_assert(!COPYW_ || (PIPE_ == PIPE_SOLO && WAVES_M_ * WAVES_N_ == 4 && KGROUPS_ == 1), "copying waves beside four computing waves: solo pipeline");
+    static_assert(PIPE != PIPE_SOLO || !BLOCK_SCALE || NW == 8 || COPYW_,
                   "solo with block scales: the accumulators have to live in the 256 vector registers of a wave");
     static_assert(PIPE == PIPE_SIMPLE || (RBA * 2) % NW == 0, "A loads must divide evenly over the waves");
     static_assert(PIPE != PIPE_SIMPLE || (TAIL == 0 && !A3), "TAIL and A3 belong to the pipelined variants");
@@ -191,7 +198,7 @@ struct GemmCfg {
     // of a step, so nothing is in flight there; the pipelined schedules live on copies in flight and would stall.
     // (The rows with two K groups keep a deep ring all the same: their copies are issued by waves of their own, and
     // the waves that read have none in flight.)
-    static_assert(KMAJ == 0 || PIPE == PIPE_SIMPLE, "K-major tiles: simple pipeline only");
+    static_assert(KMAJ == 0 || PIPE == PIPE_SIMPLE || COPYW_, "K-major tiles: simple pipeline, or copying waves");
     static_assert(!ASK_ || (BLOCK_SCALE_ && PIPE_ == PIPE_SOLO), "K-contiguous a_scale: block scales, solo pipeline");
 };
 
@@ -360,12 +367,14 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // offset of the instruction, which the buffer range check includes.
     static_assert(C::NW % 2 == 0 && C::RBA % (C::NW / 2) == 0, "A / B split of the loads must not depend on the wave");
     constexpr int LPT_A0 = C::LPT_A;                                    // loads i < LPT_A0 fetch A, the rest B
-    const int ld_r = 8 * (wave & 1) + (lane >> 3);                      // row inside the row block
+    // (GemmCfg::COPYW: the copying waves NW .. NW+3 take the places of waves 0 .. 3 in everything that follows)
+    const int lw = (C::COPYW && wave >= C::NW) ? wave - C::NW : wave;
+    const int ld_r = 8 * (lw & 1) + (lane >> 3);                        // row inside the row block
     const int ld_chunk = ((lane & 7) - ld_r) & 7;                         // rotation: see lds_slot
     // K-major tile: row block blk holds k rows 16 * (blk % (KE/16)) .. +15 of panel blk / (KE/16) (a panel = 128
     // bytes of m or n).  Bit 4 of k is bit 0 of blk = bit 1 of the wave number for every instruction of the wave
     // (NW / 2 and KE / 16 are even), so the swizzled chunk is one VGPR here too.
-    const int ld_chunk_km = (lane & 7) ^ kmajor_swz<C::ES>(ld_r + 16 * ((wave >> 1) & 1));
+    const int ld_chunk_km = (lane & 7) ^ kmajor_swz<C::ES>(ld_r + 16 * ((lw >> 1) & 1));
     const uint32_t voff_a = ld_r * p.lda + (C::KMA ? ld_chunk_km : ld_chunk) * 16;
     const uint32_t voff_b = ld_r * p.ldb + (C::KMB ? ld_chunk_km : ld_chunk) * 16;
     // K step the loop's step kt stands for (rotated start, simple pipeline only: the pipelined kernels run
@@ -383,7 +392,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     auto load_soff = [&](int i, int kt_loop) -> uint32_t {              // scalar: row block + K step
         const int kt = kpos(kt_loop);
         const bool is_a = i < LPT_A0;
-        const uint32_t blk = (wave >> 1) + (is_a ? i : i - LPT_A0) * (C::NW / 2);
+        const uint32_t blk = (lw >> 1) + (is_a ? i : i - LPT_A0) * (C::NW / 2);
         const uint32_t ld = is_a ? p.lda : p.ldb;
         if (is_a ? C::KMA : C::KMB) {
             constexpr uint32_t BPP = C::KE / 16;                        // row blocks per panel
@@ -562,7 +571,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             for (int i = 0; i < C::LPT; ++i) {
                 const bool is_a = i < LPT_A;
                 const int il = is_a ? i : i - LPT_A;
-                const uint32_t q = wave * (is_a ? LPT_A : LPT_B) + il;
+                const uint32_t q = lw * (is_a ? LPT_A : LPT_B) + il;
                 const uint32_t row = (q >> 1) * 16 + (q & 1) * 8 + (lane >> 3);
                 vo_copy[i] = row * (is_a ? p.lda : p.ldb) + chunk + GROUP_SPAN - (il & 3) * 1024;
             }
@@ -578,20 +587,20 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         };
         auto issue_a1 = [&](int i, int kt, int buf) {
             if constexpr (VOFF_PER_COPY) {
-                char *grp = smem + buf * C::A_BYTES + (wave * LPT_A + (i & ~3)) * 1024;
+                char *grp = smem + buf * C::A_BYTES + (lw * LPT_A + (i & ~3)) * 1024;
                 dma(ra_g, grp, vo_copy[i], (uint32_t)kt * C::BKB, i & 3);
             } else {
-                lds_void *dst = (lds_void *)(smem + buf * C::A_BYTES + (wave + i * C::NW) * 1024);
+                lds_void *dst = (lds_void *)(smem + buf * C::A_BYTES + (lw + i * C::NW) * 1024);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, load_soff(i, kt), 0, 0);
             }
         };
         auto issue_b1 = [&](int i, int kt) {
             if constexpr (VOFF_PER_COPY) {
                 const int il = i - LPT_A;
-                char *grp = smem + B_BASE + (kt & 1) * C::B_BYTES + (wave * LPT_B + (il & ~3)) * 1024;
+                char *grp = smem + B_BASE + (kt & 1) * C::B_BYTES + (lw * LPT_B + (il & ~3)) * 1024;
                 dma(rb_g, grp, vo_copy[i], (uint32_t)kt * C::BKB, il & 3);
             } else {
-                lds_void *dst = (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (wave + i * C::NW) * 1024 - C::A_BYTES);
+                lds_void *dst = (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (lw + i * C::NW) * 1024 - C::A_BYTES);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, load_soff(i, kt), 0, 0);
             }
         };
@@ -694,7 +703,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             };
             // 4 waves: 256 accumulator registers per lane, pinned in place (see mma128_inplace); the two
             // halves of a 16-byte MFMA pair are then issued a row apart.  8 waves: compiler-managed.
-            constexpr bool PINNED = C::NW == 4;
+            constexpr bool PINNED = C::NW == 4 && !C::COPYW;
             constexpr int HALVES = (PINNED && C::ARITH != AR_F8) ? 2 : 1;
             auto mma = [&](int a, int b, int half) {
                 if constexpr (PINNED)
@@ -708,7 +717,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // copy of the body cost register spills of its own).
             auto step = [&](int kt, int par) {             // par = kt & 1
                 const int a_nx = next_buf(a_rd);
-                constexpr bool copies = true;
+                constexpr bool copies = !C::COPYW;            // (the copying waves' loop is below)
                 // block scales of this step (fetched one step ahead) and the fetch for the next one, in front of
                 // this step's copies: by the time they are used nothing older is still in flight
                 // block scales: fetch_scales brings the a_scale rows of step kt+1 (in front of this step's
@@ -813,12 +822,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 a_rd = a_nx;
                 a_wr = next_buf(a_wr);
             };
-            if (nk > 0) {
-                if constexpr (C::BLOCK_SCALE) {
-                    fetch_a_scales(0, 0);
-                    fetch_b_scales(0);
-                    rotate_scales(0);
-                }
+            auto first_copies = [&]() {
 #pragma unroll
                 for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
 #pragma unroll
@@ -829,6 +833,49 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #pragma unroll
                     for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 1);
                 }
+            };
+            if constexpr (C::COPYW) {
+                if (wave >= C::NW) {
+                    // The copying waves: the copies of step(), at the same places between the same barriers (two in
+                    // front of the loop, one per step, one behind the loop).  A(kt+2) goes out in front of the barrier
+                    // of step kt, into the buffer of A(kt-1), which every computing wave has read before the barrier
+                    // of step kt-1; then the wait for everything older, A(kt+1) and B(kt+1), which are first read
+                    // behind this barrier; B(kt+2) goes out behind it, into the buffer of B(kt), which is in
+                    // registers everywhere since the last row of step kt-1.
+                    if (nk > 0) {
+                        first_copies();
+                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                        phase_barrier();
+                        phase_barrier();
+                        int aw = 2;
+                        for (int kt = 0; kt < nk; ++kt) {
+                            if (kt + 2 < nk) {
+#pragma unroll
+                                for (int i = 0; i < LPT_A; ++i) issue_a1(i, kt + 2, aw);
+                                __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
+                            } else {
+                                __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                            }
+                            phase_barrier();
+                            if (kt + 2 < nk) {
+#pragma unroll
+                                for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, kt + 2);
+                            }
+                            aw = next_buf(aw);
+                        }
+                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                        phase_barrier();
+                    }
+                    return;
+                }
+            }
+            if (nk > 0) {
+                if constexpr (C::BLOCK_SCALE) {
+                    fetch_a_scales(0, 0);
+                    fetch_b_scales(0);
+                    rotate_scales(0);
+                }
+                if constexpr (!C::COPYW) first_copies();
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
                 phase_barrier();
 #pragma unroll
@@ -1419,7 +1466,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         char *cwave = Cz + ((size_t)wrow0 * p.ldc + wcol0) * ES;
         // Accumulators pinned in the accumulation registers (4-wave solo pipeline) are fetched from there one
         // slab at a time; left to itself the compiler moves all 256 of them into vector registers first.
-        constexpr bool ACC_PINNED = C::PIPE == PIPE_SOLO && C::NW == 4;
+        constexpr bool ACC_PINNED = C::PIPE == PIPE_SOLO && C::NW == 4 && !C::COPYW;
         auto acc_tile = [&](int a, int b) {
             if constexpr (ACC_PINNED) {
                 acc_t t;

@@ -135,12 +135,16 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2560, 2560, 2560) == "128x128_w2x2_dma"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x2_solo"
     assert plan(Q.DT_BF16, 0, 0, 512, 4096, 4096) == "64x128_w1x4_k2"
+    # one round of 256 x 128 tiles where 256 x 256 tiles would leave half of the CUs idle: the row with copying waves
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2048, 4096, 4096) == "256x128_w2x2_cw"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 1024, 8192, 8192) == "256x128_w2x2_cw_ks"
+    assert plan(Q.DT_BF16, 0, 0, 1536, 4096, 4096) == "256x128_w2x2_cw"
     # a partly empty last round of 256 x 256 tiles: its rows become a second launch with smaller tiles
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 6144, 6144) == "256x256_w2x2_solo+128x128_w2x2_dma"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 6144, 6144) == "256x256_w2x2_solo+256x128_w2x2_cw"
     # (block scales as this layout passes them: the twin for the first launch, the simple pipeline takes any strides;
-    # 6144^3: 222 us in two launches against 231 in one)
+    # 6144^3: 210 us in two launches against 229 in one)
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 2560, 7680, 2048) == "256x256_w2x4_solo8_ks+128x128_w2x2_k2"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 6144, 6144) == "256x256_w2x4_solo8_ks+128x128_w2x2_k2"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 6144, 6144) == "256x256_w2x4_solo8_ks+256x128_w2x2_cw_ks"
     # ... also when a single launch would take smaller tiles for everything, and with a rest of at most 128 rows
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 5000, 4096, 7168) == "256x256_w2x2_solo+128x128_w2x2_k2"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 7000, 7168, 2048) == "256x256_w2x2_solo+skinny_128x32_k8"
@@ -153,7 +157,7 @@ def test_plan_names_the_kernel_without_a_device():
         Q.set_option("row_split", 1)
     # operands stored K-major: read as stored where that is cheaper than transposing, else transposed first
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 2048, 2048, 2048) == "128x128_w2x2_k2_tn"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 4096, 2048, 2048) == "128x128_w2x2_dma_tn"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 4096, 2048, 2048) == "256x128_w2x2_cw_tn"
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 6144, 4608, 7168) == "transpose+256x256_w2x4_solo8"
     assert plan(Q.DT_BF16, 0, 2, 1024, 1024, 1024) == "64x128_w1x4_k2_nn"
     assert plan(Q.DT_BF16, 0, 2, 8192, 8192, 8192) == "transpose+256x256_w2x2_solo"
