@@ -133,7 +133,7 @@ def cpu_baseline(a_q, b_q, sa, sb, rows):
 # the shapes of the reference's report (TechniqueReport.md:117-121, 151-155) and a few that do not tile evenly
 SWEEP_SHAPES = [(1024, 512, 2048), (2048, 2048, 2048), (4096, 4096, 4096), (8192, 4096, 2048), (8192, 4096, 4096),
                 (8192, 8192, 8192), (6144, 6144, 6144), (6144, 4608, 7168), (4096, 14336, 4096), (4000, 4000, 4096),
-                (512, 4096, 4096), (2048, 2048, 8192),
+                (512, 4096, 4096), (2048, 2048, 8192), (2048, 4096, 4096), (1024, 8192, 8192),
                 # row counts that are whatever a batch holds, against weight shapes
                 (1000, 4096, 4096), (3000, 8192, 4096), (5000, 4096, 7168), (7000, 7168, 2048), (200, 7168, 4096)]
 
