@@ -844,7 +844,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     // registers everywhere since the last row of step kt-1.
                     if (nk > 0) {
                         first_copies();
-                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                        // (step 0 needs A(0) and B(0); A(1) and B(1) are waited for in front of its barrier)
+                        if (nk > 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(C::LPT));
+                        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
                         phase_barrier();
                         phase_barrier();
                         int aw = 2;
