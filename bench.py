@@ -528,6 +528,18 @@ def main():
         us = _graph_time([lambda: Q.scaled_gemm(am, bm_, asm_, bsm_, cm, mm, nm_, km, Q.SCALE_BLOCK128)] * 8)
         extra["mid_fp8_block_2048x2048x8192"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * km / us / 1e6,
                                                  "frac_of_peak": 2.0 * mm * nm_ * km / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
+        # one round of 256 x 128 tiles (the row with copying waves): 2048 x 4096 x 4096, per-matrix and block scales
+        nw_, kw_ = 4096, 4096
+        aw_, saw_ = _quant_fp8(torch.randn(mm, kw_, device=dev)); bw_, sbw_ = _quant_fp8(torch.randn(nw_, kw_, device=dev))
+        cw_ = torch.empty(mm, nw_, dtype=torch.bfloat16, device=dev)
+        us = _graph_time([lambda: Q.scaled_gemm(aw_, bw_, saw_, sbw_, cw_, mm, nw_, kw_, Q.SCALE_PER_MATRIX)] * 8)
+        extra["mid_fp8_2048x4096x4096"] = {"us_per_launch": us, "tflops": 2.0 * mm * nw_ * kw_ / us / 1e6,
+                                           "frac_of_peak": 2.0 * mm * nw_ * kw_ / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
+        asw_ = (torch.rand(mm, kw_ // 128, device=dev) + 0.5) / 448; bsw_ = (torch.rand(nw_ // 128, kw_ // 128, device=dev) + 0.5) / 448
+        us = _graph_time([lambda: Q.scaled_gemm(aw_, bw_, asw_, bsw_, cw_, mm, nw_, kw_, Q.SCALE_BLOCK128)] * 8)
+        extra["mid_fp8_block_2048x4096x4096"] = {"us_per_launch": us, "tflops": 2.0 * mm * nw_ * kw_ / us / 1e6,
+                                                 "frac_of_peak": 2.0 * mm * nw_ * kw_ / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
+        del aw_, bw_, cw_
         ab16, bb16 = torch.randn(mm, km, device=dev).bfloat16(), torch.randn(nm_, km, device=dev).bfloat16()
         us = _graph_time([lambda: Q.bf16_mm(ab16, bb16, cm)] * 8)
         extra["mid_bf16_2048x2048x8192"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * km / us / 1e6,
