@@ -263,6 +263,44 @@ def stream_sweep(Q, torch, dev):
     return rows
 
 
+MID_ROWS = (160, 256, 512, 768, 1024, 1536, 2048, 2560, 3072)
+MID_WEIGHTS = ((4096, 4096), (14336, 4096), (4096, 14336), (7168, 2048), (2048, 7168), (8192, 8192))      # N x K
+
+
+def mid_sweep(Q, torch, dev):
+    """Mid-size row counts against weight shapes (9 x 6 shapes, fp8 per-matrix and bf16): this library and the vendor
+    library, each as a replayed graph of eight launches on resident operands, so that torch's dispatch does not count.
+    Microseconds per launch."""
+    rows = []
+    for fam in ("fp8", "bf16"):
+        for (N, K) in MID_WEIGHTS:
+            if fam == "fp8":
+                b, sb = _quant_fp8(torch.randn(N, K, device=dev))
+            else:
+                b = torch.randn(N, K, device=dev).bfloat16()
+            for M in MID_ROWS:
+                c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+                if fam == "fp8":
+                    a, sa = _quant_fp8(torch.randn(M, K, device=dev))
+                    ours = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)
+                    theirs = lambda: torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+                else:
+                    a = torch.randn(M, K, device=dev).bfloat16()
+                    ours = lambda: Q.bf16_mm(a, b, c)
+                    theirs = lambda: torch.matmul(a, b.t(), out=c)
+                row = {"type": fam, "M": M, "N": N, "K": K}
+                t_ours = _graph_time([ours] * 8, reps=5)
+                row.update({"this_library_us": round(t_ours, 1), "kernel": Q.last_config()})
+                try:
+                    t_theirs = _graph_time([theirs] * 8, reps=5)
+                    row.update({"vendor_us": round(t_theirs, 1), "ratio": round(t_ours / t_theirs, 3)})
+                except Exception as e:                  # a vendor row that does not run is reported, not hidden
+                    row["error"] = str(e)[:200]
+                rows.append(row)
+                print("[mid]", json.dumps(row), file=sys.stderr, flush=True)
+    return rows
+
+
 def skinny_probe(Q, torch, dev):
     """Where a launch of the skinny-M kernel spends its time (config 5 shapes, fp8):
       * graph-replay time per launch with B resident against the number of 32-column strips (= workgroups), K and
@@ -333,6 +371,9 @@ def main():
     ap.add_argument("--stream-sweep", action="store_true",
                     help="only time decode-size shapes whose weights are streamed out of HBM, this library and the vendor "
                          "library from replayed graphs, print one JSON line and exit")
+    ap.add_argument("--mid-sweep", action="store_true",
+                    help="only time 160 ... 3072 rows against six weight shapes, this library and the vendor library from "
+                         "replayed graphs, print one JSON line and exit")
     ap.add_argument("--shape", default="",
                     help="only run this library on one shape, e.g. fp8:2048x2048x8192 (fp8 | fp8block | int8 | bf16 | fp16), "
                          "--steps launches from a replayed graph; print one JSON line and exit")
@@ -367,6 +408,9 @@ def main():
         return 0
     if args.vendor_sweep:
         print(json.dumps({"vendor_sweep": vendor_sweep(Q, torch, dev)}))
+        return 0
+    if args.mid_sweep:
+        print(json.dumps({"mid_sweep": mid_sweep(Q, torch, dev)}))
         return 0
     if args.skinny_probe:
         print(json.dumps({"skinny_probe": skinny_probe(Q, torch, dev)}))
