@@ -728,63 +728,55 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 v4f part[BEHIND + 1];
                 fetch_a_scales(kt + 1, par ^ 1);
                 fetch_b_scales(kt + 1);
+                // Order of the MFMAs of a step: row by row.  With copying waves (one computing wave per SIMD, four MFMAs
+                // to a row) and block scales the last two rows go column by column instead, (TM-2, b), (TM-1, b),
+                // B(kt+1)[b]: read behind the last row's own four MFMAs, the first B fragment of the next step is
+                // wanted three MFMAs after its read is issued; this way it is seven.  (1 - 2.4 % on four shapes with
+                // block scales, whose wave has the fold to issue as well; nothing measurable without.)
+                constexpr bool JOINT = C::COPYW && C::BLOCK_SCALE;
+                constexpr int NT = TMs * C::TN, J0 = (TMs - 2) * C::TN;
+                static_assert(!JOINT || BR == TMs - 2, "the joint rows start at the barrier");
+                auto row_of_tile = [&](int i) { return (JOINT && i >= J0) ? TMs - 2 + ((i - J0) & 1) : i / C::TN; };
+                auto col_of_tile = [&](int i) { return (JOINT && i >= J0) ? (i - J0) >> 1 : i % C::TN; };
                 auto fold = [&](int i) {
                     if constexpr (C::BLOCK_SCALE) {
-                        const int pa = i / C::TN, pb = i % C::TN;
+                        const int pa = row_of_tile(i), pb = col_of_tile(i);
                         const float f = sc[pa % 2][(pb * 16) / 128];
 #pragma unroll
                         for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[i % (BEHIND + 1)][r] * f;
                     }
                 };
-#pragma unroll
-                for (int a = 0; a < TMs; ++a) {
-                    if (a == BR) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        // lgkmcnt(0) and vmcnt(LPT_A): all but the A copies of this step
-                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A) & 0xF0FF);
-                        phase_barrier();
+                // the side instructions of a row go between its MFMAs, one at a time: a run of them in front
+                // of the row would leave the matrix core idle once they take longer than one MFMA
+                auto side = [&](int a, int slot) {   // slot 0 .. TN-1: what rides behind MFMA `slot` of row a
+                    if (slot < 2) {                  // the two halves of the A fragment AHEAD rows ahead
+                        const int an = a + AHEAD;
+                        const int buf = an < TMs ? a_rd : a_nx, ar = an < TMs ? an : an - TMs;
+                        far[an % RING][slot] = frag_a(smem + buf * C::A_BYTES, ar, slot);
+                        return;
                     }
-                    // the side instructions of a row go between its MFMAs, one at a time: a run of them in front
-                    // of the row would leave the matrix core idle once they take longer than one MFMA
-                    auto side = [&](int slot) {      // slot 0 .. TN-1: what rides behind MFMA `slot` of this row
-                        if (slot < 2) {              // the two halves of the A fragment AHEAD rows ahead
-                            const int an = a + AHEAD;
-                            const int buf = an < TMs ? a_rd : a_nx, ar = an < TMs ? an : an - TMs;
-                            far[an % RING][slot] = frag_a(smem + buf * C::A_BYTES, ar, slot);
-                            return;
-                        }
-                        if (!copies) return;
-                        if (a < COPY_ROWS_A) {
+                    if (!copies) return;
+                    if (a < COPY_ROWS_A) {
 #pragma unroll
-                            for (int j = (slot - 2) * CPS_A; j < (slot - 1) * CPS_A; ++j)
-                                if (j < CPR_A && a * CPR_A + j < LPT_A) issue_a1(a * CPR_A + j, kt + 2, a_wr);
-                        } else if (a >= BR) {
-                            const int r = a - BR;
+                        for (int j = (slot - 2) * CPS_A; j < (slot - 1) * CPS_A; ++j)
+                            if (j < CPR_A && a * CPR_A + j < LPT_A) issue_a1(a * CPR_A + j, kt + 2, a_wr);
+                    } else if (a >= BR) {
+                        const int r = a - BR;
 #pragma unroll
-                            for (int j = (slot - 2) * CPS_B; j < (slot - 1) * CPS_B; ++j)
-                                if (j < CPR_B && r * CPR_B + j < LPT_B) issue_b1(LPT_A + r * CPR_B + j, kt + 2);
-                        }
-                    };
-                    if constexpr (C::BLOCK_SCALE) {
-                        // each MFMA starts from zero and gives the partial product of one 128-wide K block; it is
-                        // folded into the running sum, scaled, two MFMAs later, so the four FMAs of a tile run
-                        // under the MFMAs of the next two (hip_mix_gemm_kernel.cpp:231-244)
+                        for (int j = (slot - 2) * CPS_B; j < (slot - 1) * CPS_B; ++j)
+                            if (j < CPR_B && r * CPR_B + j < LPT_B) issue_b1(LPT_A + r * CPR_B + j, kt + 2);
+                    }
+                };
+                auto step_barrier = [&]() {
+                    __builtin_amdgcn_sched_barrier(0);
+                    // lgkmcnt(0) and vmcnt(LPT_A): all but the A copies of this step
+                    __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A) & 0xF0FF);
+                    phase_barrier();
+                };
+                if constexpr (PINNED) {
 #pragma unroll
-                        for (int b = 0; b < C::TN; ++b) {
-                            const int i = a * C::TN + b;
-                            part[i % (BEHIND + 1)] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1],
-                                                                      v4f{0, 0, 0, 0});
-                            side(b);
-                            if (b == 1) {        // factor of this row, first used behind the next MFMA
-#pragma unroll
-                                for (int j = 0; j < NBS; ++j) sc[a % 2][j] = NBS == 1 ? as_b[a] : as_b[a] * bs_c[j];
-                            }
-                            __builtin_amdgcn_sched_barrier(0);
-                            if (i >= BEHIND) fold(i - BEHIND);
-                            __builtin_amdgcn_sched_barrier(0);
-                            if (a == TMs - 1) rd_b(kt + 1, b);
-                        }
-                    } else {
+                    for (int a = 0; a < TMs; ++a) {
+                        if (a == BR) step_barrier();
 #pragma unroll
                         for (int h = 0; h < HALVES; ++h) {
 #pragma unroll
@@ -794,9 +786,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                                 // second one where a tile takes two: 16-cycle MFMAs leave room for little more
                                 // than one of them with its address arithmetic)
                                 if constexpr (HALVES == 2) {
-                                    if ((h * C::TN + b) % 2 == 0) side((h * C::TN + b) / 2);
+                                    if ((h * C::TN + b) % 2 == 0) side(a, (h * C::TN + b) / 2);
                                 } else {
-                                    side(b);
+                                    side(a, b);
                                 }
                                 // B(kt)[b] is dead: its registers take B(kt+1)[b] (where a tile takes two MFMAs:
                                 // each half as soon as its MFMA of the last row is out, so the first halves, which
@@ -811,8 +803,38 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                                 }
                             }
                         }
+                        __builtin_amdgcn_sched_barrier(0);
                     }
-                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NT; ++i) {
+                        const int a = row_of_tile(i), b = col_of_tile(i);
+                        if (i == BR * C::TN) step_barrier();
+                        if constexpr (C::BLOCK_SCALE) {
+                            // each MFMA starts from zero and gives the partial product of one 128-wide K block; it is
+                            // folded into the running sum, scaled, two MFMAs later, so the four FMAs of a tile run
+                            // under the MFMAs of the next two (hip_mix_gemm_kernel.cpp:231-244)
+                            part[i % (BEHIND + 1)] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1],
+                                                                      v4f{0, 0, 0, 0});
+                            side(a, b);
+                            // the factor of a row is formed behind the MFMA that follows the row's first one: it is first
+                            // used one MFMA later, and its register was last used (row a-2) one MFMA earlier at the latest
+                            const int fr = (JOINT && i >= J0) ? (i == J0 + 1 ? TMs - 2 : (i == J0 + 2 ? TMs - 1 : -1)) : (b == 1 ? a : -1);
+                            if (fr >= 0) {
+#pragma unroll
+                                for (int j = 0; j < NBS; ++j) sc[fr % 2][j] = NBS == 1 ? as_b[fr] : as_b[fr] * bs_c[j];
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                            if (i >= BEHIND) fold(i - BEHIND);
+                            __builtin_amdgcn_sched_barrier(0);
+                        } else {
+                            mma(a, b, 0);
+                            side(a, b);
+                        }
+                        // B(kt)[b] is dead after its MFMA of the last row: its registers take B(kt+1)[b]
+                        if (a == TMs - 1) rd_b(kt + 1, b);
+                        if (i == NT - 1 || (!(JOINT && i >= J0) && b == C::TN - 1)) __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
                 if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
