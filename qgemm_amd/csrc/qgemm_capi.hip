@@ -251,10 +251,11 @@ bool mfma_shape_ok(const NtProblem &q) {
 // 256 x 256 tile (one per CU), 0.85 us for 128 x 128 with two per CU and 0.66 us alone, 0.43 us for the 128 x 128
 // row with two K groups (one per CU: it only wins where there are no more tiles than CUs; 2048 x 2048 x 2048 / 8192
 // 12.1 / 32.5 us), 0.52 us for 64 x 128 and 0.27 us for its row with two K groups (512 x 4096 x 4096 13.5 us, two
-// rounds of 64 steps 44 us), 0.39 us for 128 x 32; 0.70 us for 256 x 128 with its copying waves, which is what the
-// 256 x 256 tile needs per flop, and 6.5 - 8 us around a single round (2048 x 4096 x 4096 30.6 us, 1024 x 8192 x 8192
-// 52.7, 2048 x 3584 x 2048 17.1; it wins where its tiles make one round of CUs and the 256 x 256 tiles would leave
-// half of them idle: 6 - 17 % over the two-stage 128 x 128 row there, with block scales up to 24 %).
+// rounds of 64 steps 44 us), 0.39 us for 128 x 32; for 256 x 128 with its copying waves 0.71 us with every CU at work,
+// which is what the 256 x 256 tile needs per flop, and 0.58 us with 160 - 224 tiles (0.93 / 0.76 with block scales),
+// plus 6 us around a round (2048 x 4096 x 4096 29.3 us, 1024 x 8192 x 8192 50.8, 1536 x 4096 x 4096 25.2,
+// 768 x 7168 x 2048 14.8; it wins where its tiles make one round of CUs and the 256 x 256 tiles would leave half of
+// them idle: 6 - 17 % over the two-stage 128 x 128 row there, with block scales up to 24 %).
 // A K split adds 4 us and the partial planes at 3 TB/s.
 //
 // M <= 64 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
@@ -277,7 +278,7 @@ struct TileModel {
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.32, 1.04},
                                  {128, 128, 1, 0.43, 0.43, 4.5, true, 1, 0.50, 0.50},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
                                  {64, 128, 1, 0.27, 0.27, 4.5, true, 1, 0.34, 0.34},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60},
-                                 {256, 128, 1, 0.70, 0.70, 6.5, false, 1, 0.98, 0.98}};
+                                 {256, 128, 1, 0.71, 0.58, 6.0, false, 1, 0.93, 0.76}};
 // rows with two K groups: two sets of computing waves on a tile that otherwise has one (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 

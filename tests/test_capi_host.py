@@ -132,7 +132,8 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 1536, 1536, 1536) == "128x128_w2x2_k2"
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 2048, 2048, 8192) == "128x128_w2x2_k2"
     assert plan(Q.DT_BF16, 0, 0, 512, 8192, 8192) == "128x128_w2x2_k2"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2560, 2560, 2560) == "128x128_w2x2_dma"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2560, 2560, 2560) == "256x128_w2x2_cw"       # 200 tiles: 19.1 us, 128 x 128: 21.0
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 4096, 2048, 2048) == "128x128_w2x2_dma"      # 256 tiles, 16 K steps: 18.1 / 18.8 either way
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x2_solo"
     assert plan(Q.DT_BF16, 0, 0, 512, 4096, 4096) == "64x128_w1x4_k2"
     # one round of 256 x 128 tiles where 256 x 256 tiles would leave half of the CUs idle: the row with copying waves
