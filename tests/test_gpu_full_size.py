@@ -291,3 +291,49 @@ def test_row_split_with_a_short_rest_and_against_smaller_tiles(shape, m_main, re
     assert "+" in name, name
     ref = R.gemm_f32acc(R.decode_fp8(qa8[rows]), R.decode_fp8(qb8)) * np.float32(sa * sb)
     assert_close(host(cb)[rows], ref, what=name)
+
+
+def test_one_round_of_256x128_tiles_int8_and_block_scales():
+    """2048 x 4096 x 4096, a shape the heuristic gives to the row with copying waves (256 tiles of 256 x 128): int32
+    accumulators identical over the whole matrix to those of a 128 x 128 tile and of a K split, and bit-exact
+    against the oracle on sampled rows and columns; with 128-block scales, sampled rows against the oracle and an
+    exact factor of four when every a_scale is doubled and every b_scale too."""
+    M, N, K = 2048, 4096, 4096
+    say("one round of 256x128 tiles", (M, N, K))
+    qa, sa = R.quantize_int8(R.fill_normal((M, K), 52))
+    qb, sb = R.quantize_int8(R.fill_normal((N, K), 53))
+    da, db_ = dev(qa), dev(qb)
+    c = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    Q.int8_mm(da, db_, scalar(sa), scalar(sb), c)
+    assert Q.last_config() == "256x128_w2x2_cw", Q.last_config()
+    got = host(c)
+    rows, cols = _sample(M, 32, 3), _sample(N, 32, 4)
+    assert np.array_equal(got[rows], R.gemm_i8_i32(qa[rows], qb))
+    assert np.array_equal(got[:, cols], R.gemm_i8_i32(qa, qb[cols]))
+    for force, split in ((2, 1), (24, 2)):
+        Q.set_option("force_config", force)
+        Q.set_option("force_split", split)
+        c2 = torch.zeros_like(c)
+        Q.int8_mm(da, db_, scalar(sa), scalar(sb), c2)
+        assert torch.equal(c, c2), Q.last_config()
+    Q.set_option("force_config", -1)
+    Q.set_option("force_split", 0)
+    # block scales
+    rng = np.random.default_rng(54)
+    a8 = R.encode_fp8(np.clip(R.fill_normal((M, K), 55), -4, 4))
+    b8 = R.encode_fp8(np.clip(R.fill_normal((N, K), 56), -4, 4))
+    as_ = (0.5 + rng.random((M, K // 128))).astype(np.float32)
+    bs = (0.5 + rng.random((N // 128, K // 128))).astype(np.float32)
+    ta, tb = fp8_tensor(a8), fp8_tensor(b8)
+    cf = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    Q.scaled_gemm(ta, tb, dev(as_), dev(bs), cf, M, N, K, Q.SCALE_BLOCK128)
+    assert Q.last_config() == "256x128_w2x2_cw_ks", Q.last_config()
+    gotf = host(cf)
+    rows = _sample(M, 8, 5)
+    ref = R.gemm_fp8_block(R.decode_fp8(a8[rows]), R.decode_fp8(b8), as_[rows], bs)
+    # (every kernel of the library lands within 4.2e-3 of the exact sums here, rms 9e-4 at |C| around 55: that is the
+    # MFMA's own accumulation of 128 products, the fp32 oracle is within 6e-5; the stated tolerance covers it)
+    assert_close(gotf[rows], ref, what=Q.last_config())
+    cf4 = torch.zeros_like(cf)
+    Q.scaled_gemm(ta, tb, dev(2 * as_), dev(2 * bs), cf4, M, N, K, Q.SCALE_BLOCK128)
+    assert torch.equal(cf4, 4 * cf)
