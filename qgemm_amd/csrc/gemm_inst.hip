@@ -148,6 +148,21 @@ static const Variant kTable[] = {
 #else
     ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
 #endif
+    // 192 x 256 on the 8-wave solo schedule (96 x 64 wave tiles): for row counts whose 256-row tiles would leave
+    // a round of CUs partly empty (3072 rows against 4096 columns: 256 tiles instead of 192), and its twin for
+    // K-contiguous a_scale.  K-contiguous operands only.
+#if INST_KMAJ
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+#else
+    ROWP("192x256_w2x4_solo8", 192, 256, 2, 4, LOAD_DMA, PIPE_SOLO, true),
+#if INST_BLOCK
+    row_of<true, GemmCfg<INST_ARITH, true, 192, 256, 2, 4, LOAD_DMA, PIPE_SOLO, 0, true, 0, 0, 1, true>,
+           CFG(128, 128, 2, 2, LOAD_DMA, PIPE_SIMPLE)>("192x256_w2x4_solo8_ks", false),
+#else
+    ROW("128x128_w2x2_dma", 128, 128, 2, 2, LOAD_DMA, false),
+#endif
+#endif
 };
 
 const Variant *INST_FN(int *count) {

@@ -182,8 +182,9 @@ struct GemmCfg {
     static_assert(!BLOCK_SCALE || (128 % WN == 0 || WN % 128 == 0), "wave tile must align with 128-wide scale blocks");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS is 160 KiB per CU");
     static_assert(PIPE != PIPE_PINGPONG || (NW == 8 && LOADER == LOAD_DMA), "ping-pong needs 8 waves and the DMA loader");
-    static_assert(PIPE != PIPE_SOLO || ((NW == 4 || NW == 8) && LOADER == LOAD_DMA && A3 && TM % 4 == 0 && TM >= 8 && TN >= 4),
-                  "solo: 4 or 8 waves, DMA loader, A triple-buffered, at least 8 rows of at least 4 MFMAs per step");
+    static_assert(PIPE != PIPE_SOLO || ((NW == 4 || NW == 8) && LOADER == LOAD_DMA && A3 && TN >= 4 &&
+                                        ((TM % 4 == 0 && TM >= 8) || (TM == 6 && NW == 8))),
+                  "solo: 4 or 8 waves, DMA loader, A triple-buffered, at least 8 rows (8 waves: or 6) of at least 4 MFMAs per step");
     static_assert(!COPYW_ || (PIPE_ == PIPE_SOLO && WAVES_M_ * WAVES_N_ == 4 && KGROUPS_ == 1), "copying waves beside four computing waves: solo pipeline");
     static_assert(PIPE != PIPE_SOLO || !BLOCK_SCALE || NW == 8 || COPYW_,
                   "solo with block scales: the accumulators have to live in the 256 vector registers of a wave");
@@ -551,14 +552,13 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         // registers to spare) and the scalar offset is the K step alone, one register for all copies of a step;
         // with one wave per SIMD every scalar add between two MFMAs is issue time the MFMAs do not get (with two
         // waves per SIMD it still pays: int8 -1.8 %, fp8 -1.4 %, bf16 -0.8 % on 8192^3; block scales unchanged).
-        constexpr bool VOFF_PER_COPY = C::PIPE == PIPE_SOLO && C::KMAJ == 0;
+        constexpr bool VOFF_PER_COPY = C::PIPE == PIPE_SOLO && C::KMAJ == 0 && LPT_A % 4 == 0 && LPT_B % 4 == 0;
         // ... and a wave's copies are neighbours in LDS (instruction q = wave * LPT_A + i of the A list, likewise
         // for B; elsewhere q = wave + i * NW), so that four of them share one LDS base in M0 and differ in the
         // instruction's immediate offset (0 .. 3072).  The hardware adds that immediate to the global address as
         // well: the descriptors of these kernels start GROUP_SPAN bytes below the tile and every vector offset
         // carries GROUP_SPAN minus its immediate, so no offset is negative and the range check sees the same sums.
         constexpr int GROUP_SPAN = 3072;
-        static_assert(!VOFF_PER_COPY || (LPT_A % 4 == 0 && LPT_B % 4 == 0), "copies go in groups of four");
         uint32_t vo_copy[VOFF_PER_COPY ? C::LPT : 1];
         __amdgpu_buffer_rsrc_t ra_g = ra, rb_g = rb;
         if constexpr (VOFF_PER_COPY) {
@@ -621,7 +621,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             constexpr int COPY_ROWS_A = 4, CPR_A = (LPT_A + COPY_ROWS_A - 1) / COPY_ROWS_A;   // A copies per row
             // A fragment ring: row a lives in slot a % RING and is read AHEAD rows before it is used (one row
             // ahead is less than the LDS latency under load: the wave then waits in front of every row).
-            constexpr int RING = 4, AHEAD = RING / 2;
+            // (wave tiles of six row blocks, the 192-row tile: three slots; a read then lands in the slot of the row
+            // whose last MFMA has just been issued)
+            constexpr int RING = TMs % 4 == 0 ? 4 : 3, AHEAD = 2;
             constexpr int BR = TMs - AHEAD;                  // row the barrier stands in front of
             constexpr int CPR_B = (LPT_B + AHEAD - 1) / AHEAD;                              // B copies per row
             constexpr int SLOTS = C::TN - 2;                 // MFMAs of a row a copy can ride behind

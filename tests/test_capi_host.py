@@ -98,7 +98,11 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F16, 0, 0, 1024, 1024, 512) == "128x32_w4x1_dma"                        # (8 K steps: one per wave)
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4096) == "256x256_w2x2_solo"     # config 2
     # int8 and 16-bit types: 4 waves when the tiles fill whole rounds of CUs, 8 waves in a partly filled round
-    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x4_solo8"
+    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 3840, 4096, 4096) == "256x256_w2x4_solo8"
+    # a partly filled round that 192-row tiles fill better: 3072^3 is 144 tiles of 256 x 256 or 192 of 192 x 256
+    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "192x256_w2x4_solo8"
+    assert plan(Q.DT_BF16, 0, 0, 3072, 4096, 4096) == "192x256_w2x4_solo8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 1536, 7168, 2048) == "192x256_w2x4_solo8_ks"
     assert plan(Q.DT_BF16, 0, 0, 8192, 4096, 4096) == "256x256_w2x2_solo"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "256x256_w2x2_solo"  # config 3
     # config 4: the twin of the 8-wave kernel that reads a_scale as this layout passes it (56 K blocks per row: even)
@@ -134,7 +138,8 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_BF16, 0, 0, 512, 8192, 8192) == "128x128_w2x2_k2"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2560, 2560, 2560) == "256x128_w2x2_cw"       # 200 tiles: 19.1 us, 128 x 128: 21.0
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 4096, 2048, 2048) == "128x128_w2x2_dma"      # 256 tiles, 16 K steps: 18.1 / 18.8 either way
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "256x256_w2x2_solo"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 3072, 3072, 3072) == "192x256_w2x4_solo8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 3840, 4096, 4096) == "256x256_w2x2_solo"
     assert plan(Q.DT_BF16, 0, 0, 512, 4096, 4096) == "64x128_w1x4_k2"
     # one round of 256 x 128 tiles where 256 x 256 tiles would leave half of the CUs idle: the row with copying waves
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 2048, 4096, 4096) == "256x128_w2x2_cw"
@@ -153,7 +158,8 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 4096, 14336, 4096) == "256x256_w2x2_solo"     # 3.5 rounds: no gain
     Q.set_option("row_split", 0)
     try:
-        assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 6144, 6144) == "256x256_w2x2_solo"
+        # (one launch: 768 tiles of 192 x 256 are three full rounds, 166 us against 187 on 256 x 256 tiles)
+        assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 6144, 6144) == "192x256_w2x4_solo8"
     finally:
         Q.set_option("row_split", 1)
     # operands stored K-major: read as stored where that is cheaper than transposing, else transposed first

@@ -69,3 +69,41 @@ def test_every_number_of_k_steps(fam):
                 assert name.replace("_ks", "").startswith(want), name
                 assert ("splitk" in name) == (split > 1), name
                 assert np.array_equal(host(c), ref), (name, ksteps, split)
+
+
+@pytest.mark.parametrize("fam", ["f8", "f8_block", "i8", "bf16"])
+def test_192_row_tile_every_number_of_k_steps(fam):
+    """The 192 x 256 row of the 8-wave solo schedule (wave tiles of six row blocks, a fragment ring of three slots,
+    three A copies and four B copies per wave and step): the same sweep over K steps, K splits and ragged tiles."""
+    for (M, N) in ((192, 256), (300, 200), (576, 512)):
+        for ksteps in (1, 2, 3, 4, 5, 6, 7, 8, 9, 13, 16):
+            for split in ((1, 2) if ksteps >= 4 else (1,)):
+                K = ksteps * (64 if fam == "bf16" else 128)
+                say("192-row tile", fam, (M, N, K), "split", split)
+                Q.set_option("force_config", 26)
+                Q.set_option("force_split", split)
+                rng = np.random.default_rng(300 * ksteps + split)
+                a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+                b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+                c = torch.full((M, N), -7.0, dtype=torch.float32, device="cuda")
+                if fam == "i8":
+                    c = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+                    Q.int8_mm(dev(a.astype(np.int8)), dev(b.astype(np.int8)), scalar(1), scalar(1), c)
+                    ref = R.gemm_i8_i32(a.astype(np.int8), b.astype(np.int8))
+                elif fam == "bf16":
+                    Q.gemm(dev(a).bfloat16(), dev(b).bfloat16(), c, "nk")
+                    ref = R.gemm_f32acc(a, b)
+                elif fam == "f8":
+                    Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), scalar(1), scalar(1), c, M, N, K,
+                                  Q.SCALE_PER_MATRIX)
+                    ref = R.gemm_f32acc(a, b)
+                else:
+                    as_ = (2.0 ** rng.integers(-3, 4, size=(M, ksteps))).astype(np.float32)
+                    bs = (2.0 ** rng.integers(-3, 4, size=((N + 127) // 128, ksteps))).astype(np.float32)
+                    Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K,
+                                  Q.SCALE_BLOCK128)
+                    ref = R.gemm_fp8_block(a, b, as_, bs)
+                name = Q.last_config()
+                assert name.replace("_ks", "").startswith("192x256_w2x4_solo8"), name
+                assert ("splitk" in name) == (split > 1), name
+                assert np.array_equal(host(c), ref), (name, ksteps, split)

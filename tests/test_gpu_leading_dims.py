@@ -34,8 +34,9 @@ def _poison_intact(whole, M, N, poison):
 
 
 # variant rows (gemm_inst.hip): 2 = 128x128 (staged epilogue), 11 = 256x256 4-wave solo, 12 = 8-wave solo,
-# 13 = 128x32 and 15 = 16x32 (no LDS staging of C), 16 = 128x128 with two K groups, 24 = 256x128 with copying waves
-EXITS = [2, 11, 12, 13, 15, 16, 24]
+# 13 = 128x32 and 15 = 16x32 (no LDS staging of C), 16 = 128x128 with two K groups, 24 = 256x128 with copying waves,
+# 26 = 192x256 (8-wave solo)
+EXITS = [2, 11, 12, 13, 15, 16, 24, 26]
 
 
 @pytest.mark.parametrize("pad", [8, 5])
@@ -76,7 +77,7 @@ def test_fp8_bf16_out_padded_ldc(pad, variant, shape):
 
 
 @pytest.mark.parametrize("pad", [8, 5])
-@pytest.mark.parametrize("variant", [2, 12, 13, 24])
+@pytest.mark.parametrize("variant", [2, 12, 13, 24, 26])
 def test_fp8_block_scaled_padded_ldc(pad, variant):
     M, N, K = 256, 384, 512
     say("ldC fp8 block", "pad", pad, "variant", variant)

@@ -14,7 +14,7 @@ from tests.util import (assert_close, dev, fp8_inputs, fp8_tensor, host, int8_in
 
 pytestmark = pytest.mark.gpu
 
-N_VARIANTS = 26         # rows of the variant table in qgemm_amd/csrc/gemm_inst.hip
+N_VARIANTS = 28         # rows of the variant table in qgemm_amd/csrc/gemm_inst.hip
 
 
 @pytest.fixture(autouse=True)

@@ -11,7 +11,7 @@ from oracle import cpu_ref as R
 from tests.util import assert_close, dev, fp8_tensor, host, say, scalar
 
 pytestmark = pytest.mark.gpu
-N_VARIANTS = 26
+N_VARIANTS = 28
 
 
 @pytest.fixture(autouse=True)
