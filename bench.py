@@ -584,6 +584,14 @@ def main():
         extra["mid_fp8_block_2048x4096x4096"] = {"us_per_launch": us, "tflops": 2.0 * mm * nw_ * kw_ / us / 1e6,
                                                  "frac_of_peak": 2.0 * mm * nw_ * kw_ / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
         del aw_, bw_, cw_
+        # a partly filled round of 256 x 256 tiles that 192-row tiles fill: 3072 x 4096 x 4096
+        mp_ = 3072
+        ap_, sap_ = _quant_fp8(torch.randn(mp_, kw_, device=dev)); bp_, sbp_ = _quant_fp8(torch.randn(nw_, kw_, device=dev))
+        cp_ = torch.empty(mp_, nw_, dtype=torch.bfloat16, device=dev)
+        us = _graph_time([lambda: Q.scaled_gemm(ap_, bp_, sap_, sbp_, cp_, mp_, nw_, kw_, Q.SCALE_PER_MATRIX)] * 8)
+        extra["mid_fp8_3072x4096x4096"] = {"us_per_launch": us, "tflops": 2.0 * mp_ * nw_ * kw_ / us / 1e6,
+                                           "frac_of_peak": 2.0 * mp_ * nw_ * kw_ / us / 1e6 / PEAK_TFLOPS["f8"], "kernel": Q.last_config()}
+        del ap_, bp_, cp_
         ab16, bb16 = torch.randn(mm, km, device=dev).bfloat16(), torch.randn(nm_, km, device=dev).bfloat16()
         us = _graph_time([lambda: Q.bf16_mm(ab16, bb16, cm)] * 8)
         extra["mid_bf16_2048x2048x8192"] = {"us_per_launch": us, "tflops": 2.0 * mm * nm_ * km / us / 1e6,
