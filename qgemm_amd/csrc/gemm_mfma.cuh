@@ -168,7 +168,9 @@ struct GemmCfg {
     // like the operands, 512 bytes per stage behind the ring, so that every copy of the loop is of one kind and the
     // wave's own count of copies in flight stays exact (a register load among them makes the compiler wait for all).
     // (or, K-contiguous a_scale: four slots of BM rows x four K blocks, see the K loop)
-    static constexpr int SCALE_LDS = (BLOCK_SCALE_ && KGROUPS_ == 2) ? (NSTAGE * 512 > 64 * BM_ ? NSTAGE * 512 : 64 * BM_) : 0;
+    // (copying waves beside the solo schedule, the twin for K-contiguous a_scale: the same four slots, see SCALES_LDS)
+    static constexpr int SCALE_LDS = (BLOCK_SCALE_ && KGROUPS_ == 2) ? (NSTAGE * 512 > 64 * BM_ ? NSTAGE * 512 : 64 * BM_)
+                                     : (BLOCK_SCALE_ && COPYW_ && ASK_) ? 64 * BM_ : 0;
     static constexpr int LDS_BYTES = (A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES) + SCALE_LDS;
     static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && (!BLOCK_SCALE || KGROUPS_ == 2) &&
                                    (KMAJ_ == 0 || KGROUPS_ == 2) && STAGES_ >= 2 && STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
@@ -647,8 +649,18 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             float as_b[TMs], bs_c[NBS], sc[2][NBS];
             v2i as_pair[NLD];
             constexpr bool as_kcont = C::ASK;
+            // Copying waves and K-contiguous a_scale (the twin `_ks` of the row with copying waves): the computing waves
+            // fetch no scales themselves.  A copying wave brings the scales of four K blocks of 64 tile rows in one
+            // 16-byte-per-lane copy, in front of the A copies of every fourth step, into slot (kt / 4) % 4 of four
+            // behind the operand buffers ([row][4 K blocks]; the host picks this twin only where rows and K slices
+            // start at multiples of four blocks), and a computing wave reads the eight values of its lane for the
+            // next step where the other kernels distribute what they fetched.  That takes the last memory instruction
+            // but the b_scale load out of the computing waves, the lane swaps with it, and a row of a_scale costs
+            // the fill path one request per four steps instead of one per two from each of the waves that share it.
+            constexpr bool SCALES_LDS = C::BLOCK_SCALE && C::COPYW && C::ASK;
+            constexpr int SC_BASE = 3 * C::A_BYTES + 2 * C::B_BYTES;
             auto fetch_a_scales = [&](int kt, int comp) {      // for K step kt (of this slice; comp = kt & 1)
-                if constexpr (C::BLOCK_SCALE) {
+                if constexpr (C::BLOCK_SCALE && !SCALES_LDS) {
                     const uint32_t kb = kbeg + kt;
                     if (as_kcont) {
                         if (comp == 0) {
@@ -674,8 +686,18 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             };
             // With one b_scale per wave tile and K block (NBS == 1) the factor a_scale * b_scale is formed here, on
             // the two registers the loads brought, instead of once per row of MFMAs: the same product, the same bits.
-            auto rotate_scales = [&](int comp) {
-                if constexpr (C::BLOCK_SCALE) {
+            auto rotate_scales = [&](int comp, int kt_next) {  // (kt_next: the step the scales are for)
+                if constexpr (SCALES_LDS) {
+                    const char *sc_ = smem + SC_BASE + ((kt_next >> 2) & 3) * (16 * C::BM) + (kt_next & 3) * 4 +
+                                      (wm * C::WM + (lane & 15)) * 16;
+#pragma unroll
+                    for (int a = 0; a < TMs; ++a) {
+                        const float x = *(const float *)(sc_ + a * 256);
+                        as_b[a] = NBS == 1 ? x * bs_raw[0] : x;
+                    }
+#pragma unroll
+                    for (int j = 0; j < NBS; ++j) bs_c[j] = bs_raw[j];
+                } else if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
                     for (int j = 0; j < NLD; ++j) {
                         unsigned x = (unsigned)as_pair[j][comp];
@@ -841,7 +863,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
                     for (int i = TMs * C::TN - BEHIND; i < TMs * C::TN; ++i) fold(i);
-                    rotate_scales(par ^ 1);
+                    rotate_scales(par ^ 1, kt + 1);
                 }
                 a_rd = a_nx;
                 a_wr = next_buf(a_wr);
@@ -866,7 +888,16 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     // of step kt-1; then the wait for everything older, A(kt+1) and B(kt+1), which are first read
                     // behind this barrier; B(kt+2) goes out behind it, into the buffer of B(kt), which is in
                     // registers everywhere since the last row of step kt-1.
+                    auto issue_scale_group = [&](int kt) {     // K steps kt .. kt + 3 of this slice, kt a multiple of four
+                        if constexpr (SCALES_LDS) {
+                            static_assert(C::BM == 64 * C::NPROD, "one copy of 64 rows per copying wave");
+                            lds_void *dst = (lds_void *)(smem + SC_BASE + ((kt >> 2) & 3) * (16 * C::BM) + lw * 1024);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ras, dst, 16, (row0 + 64 * lw + lane) * p.as_ms * 4,
+                                                                     (kbeg + (uint32_t)kt) * 4, 0, 0);
+                        }
+                    };
                     if (nk > 0) {
+                        issue_scale_group(0);
                         first_copies();
                         // (step 0 needs A(0) and B(0); A(1) and B(1) are waited for in front of its barrier)
                         if (nk > 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(C::LPT));
@@ -876,6 +907,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         int aw = 2;
                         for (int kt = 0; kt < nk; ++kt) {
                             if (kt + 2 < nk) {
+                                if (((kt + 2) & 3) == 0) issue_scale_group(kt + 2);     // older than the A copies: waited for below
 #pragma unroll
                                 for (int i = 0; i < LPT_A; ++i) issue_a1(i, kt + 2, aw);
                                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
@@ -899,11 +931,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 if constexpr (C::BLOCK_SCALE) {
                     fetch_a_scales(0, 0);
                     fetch_b_scales(0);
-                    rotate_scales(0);
+                    if constexpr (!SCALES_LDS) rotate_scales(0, 0);
                 }
                 if constexpr (!C::COPYW) first_copies();
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
                 phase_barrier();
+                if constexpr (SCALES_LDS) rotate_scales(0, 0);      // (the first group of scales is in LDS behind this barrier)
 #pragma unroll
                 for (int b = 0; b < C::TN; ++b) rd_b(0, b);
 #pragma unroll

@@ -727,9 +727,15 @@ bool settle_scale_layout(const NtProblem &q, Plan &pl) {
     // plan either takes any strides (simple and ping-pong pipelines) or has a twin for it
     const bool ks_form = q.as_ks == 1 && q.as_ms % 2 == 0 && ((uintptr_t)q.as & 7u) == 0;
     bool as_is = true;
+    // (the twin of the row with copying waves takes the scales of four K blocks per copy: rows 16-byte aligned, K and
+    // every K slice a multiple of four blocks)
+    const bool ks4_form = ks_form && q.as_ms % 4 == 0 && ((uintptr_t)q.as & 15u) == 0;
     for (const Plan *p = &pl; as_is && p; p = p->rest.get()) {
         if (p->v->a_scale_any_stride) continue;
-        as_is = ks_form && partner(p->v, true) && !(p->a.nsplit > 1 && p->a.ksteps_per_split % 2 != 0);
+        const Variant *twin = partner(p->v, true);
+        as_is = ks_form && twin && !(p->a.nsplit > 1 && p->a.ksteps_per_split % 2 != 0);
+        if (as_is && std::strstr(twin->name, "_cw"))
+            as_is = ks4_form && p->a.ksteps % 4 == 0 && !(p->a.nsplit > 1 && p->a.ksteps_per_split % 4 != 0);
     }
     for (Plan *p = &pl; p; p = p->rest.get()) {
         if (p->v->a_scale_any_stride) continue;
