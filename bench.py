@@ -35,10 +35,24 @@ PEAK_HBM_GBS = 8000.0
 # profiles/gemm_nt_f8_256x256_solo_8192.md.  Keyed by (kernel name, M): None where no counter run exists.
 FETCH_FACTOR = 2.0     # copy of 262144 KiB reads FETCH_SIZE = 131084
 WRITE_FACTOR = 1.0     # copy of 262144 KiB reads WRITE_SIZE = 262144
-MEASURED_TRAFFIC_BYTES = {      # (FETCH_SIZE KiB * factor + WRITE_SIZE KiB * factor) * 1024
-    ("256x256_w2x4_solo8", 8192): (405763.0 * FETCH_FACTOR + 131072.0 * WRITE_FACTOR) * 1024.0,
-    ("256x256_w2x2_solo", 8192): (399561.0 * FETCH_FACTOR + 131206.0 * WRITE_FACTOR) * 1024.0,
+MEASURED_TRAFFIC_BYTES = {      # (FETCH_SIZE KiB * factor + WRITE_SIZE KiB * factor) * 1024, and where the readings are kept
+    ("256x256_w2x4_solo8", 8192): ((405763.0 * FETCH_FACTOR + 131072.0 * WRITE_FACTOR) * 1024.0,
+                                   "profiles/gemm_nt_f8_256x256_solo8_8192.md"),
+    ("256x256_w2x2_solo", 8192): ((399561.0 * FETCH_FACTOR + 131206.0 * WRITE_FACTOR) * 1024.0,
+                                  "profiles/gemm_nt_f8_256x256_solo_8192.md"),
 }
+
+
+def measured_traffic(kernel, M):
+    """-> (bytes per launch or None, where the figure comes from).  The figure is a constant read off two offline
+    rocprofv3 --pmc runs, not measured by this run; a kernel without such a run says so loudly instead of a bare null."""
+    hit = MEASURED_TRAFFIC_BYTES.get((kernel, M))
+    if hit:
+        return hit[0], "constant from offline rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), %s" % hit[1]
+    print("bench.py: WARNING: no HBM traffic counters on record for kernel %r at M=%d; roofline.traffic is null. "
+          "Run the two --pmc commands of profiles/gemm_nt_f8_256x256_solo_8192.md for it and add the readings to "
+          "MEASURED_TRAFFIC_BYTES." % (kernel, M), file=sys.stderr, flush=True)
+    return None, "MISSING: no rocprofv3 --pmc run on record for kernel %s at M=%d" % (kernel, M)
 
 
 def _time_launches(fn, steps, warmup):
@@ -428,6 +442,7 @@ def main():
     tflops_wall = flops / (wall_ms * 1e-3) / 1e12
     tflops_ev = flops / (ev_ms * 1e-3) / 1e12
 
+    traffic, traffic_source = measured_traffic(cfg_name, M)
     out = {
         "metric": "scaled-GEMM TFLOP/s (fp8 e4m3 per-matrix scales, M=N=K=%d), 1 GPU" % M,
         "value": tflops_wall, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -436,7 +451,7 @@ def main():
         "config": {"workload": f"fp8-e4m3 per-matrix-scaled GEMM M=N=K={M}, A MxK and B NxK K-contiguous, bf16 out",
                    "kernel": cfg_name},
         "roofline": {"bound": "mfma", "achieved": tflops_ev, "peak": PEAK_TFLOPS["f8"], "unit": "TFLOP/s",
-                     "frac": tflops_ev / PEAK_TFLOPS["f8"], "traffic": MEASURED_TRAFFIC_BYTES.get((cfg_name, M)),
+                     "frac": tflops_ev / PEAK_TFLOPS["f8"], "traffic": traffic, "traffic_source": traffic_source,
                      "traffic_unit": "bytes per launch (L2 <-> fabric, rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
                      "algorithmic_bytes": float(M * K + N * K + 2 * M * N),
                      "kernel_ms": ev_ms, "flops_per_launch": flops},

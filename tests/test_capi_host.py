@@ -172,12 +172,12 @@ def test_plan_names_the_kernel_without_a_device():
     # K not a multiple of 128 bytes: the any-shape kernel
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 100, 100, 100) == "strided_any_shape"
     # forced rows are honoured, and a forced split shows in the name
-    Q.set_option("force_config", 2)
+    Q.force_config("128x128_w2x2_dma")
     Q.set_option("force_split", 4)
     try:
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "128x128_w2x2_dma_splitk4"
     finally:
-        Q.set_option("force_config", -1)
+        Q.force_config(None)
         Q.set_option("force_split", 0)
     with pytest.raises(Q.QgemmError):
         plan(Q.DT_I8, Q.SCALE_BLOCK128, 0, 256, 256, 256)        # block scales are fp8 only
@@ -277,3 +277,20 @@ def test_fnuz_fp8_is_refused_not_misread():
         Q.fp8_mm(ok, ok, s, s, torch.zeros((32, 16), dtype=torch.bfloat16))
     with pytest.raises(ValueError):          # c with a non-unit inner stride
         Q.fp8_mm(ok, ok, s, s, torch.zeros((32, 64), dtype=torch.bfloat16)[:, ::2])
+
+
+def test_bench_has_traffic_counters_for_the_headline_kernel():
+    """bench.py's roofline.traffic is a constant read off offline counter runs, keyed by kernel name: the kernel the
+    planner names for the headline workload has to have an entry (and the file the entry cites has to exist), or the
+    bench line would carry a null."""
+    import importlib.util
+    root = ROOT
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    name = Q.plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192)
+    traffic, source = bench.measured_traffic(name, 8192)
+    assert traffic and traffic > 2 * 8192 * 8192 + 2 * 8192 * 8192, (name, source)
+    cited = [w for w in source.replace(",", " ").split() if w.startswith("profiles/")]
+    assert cited and all(os.path.exists(os.path.join(root, f)) for f in cited), source
+    assert bench.measured_traffic("no_such_kernel", 8192)[0] is None

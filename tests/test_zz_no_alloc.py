@@ -15,11 +15,23 @@ from tests.util import dev, fp8_inputs, fp8_tensor, int8_inputs, say, scalar
 pytestmark = pytest.mark.gpu
 
 
+def _memory_state():
+    """(library workspace base, its size, free device memory): what a call that allocates would change."""
+    base, size = C.c_void_p(), C.c_size_t()
+    L.check(L.load_library().qgemm_workspace_info(C.byref(base), C.byref(size)))
+    torch.cuda.synchronize()
+    return base.value, size.value, torch.cuda.mem_get_info()[0]
+
+
 def _call(static, in_dt, scale_mode, layout, a, b, sa, sb, c, M, N, K, split):
     lib = L.load_library()
     fn = lib.qgemm_scaled_gemm_static if static else lib.qgemm_scaled_gemm
+    before = _memory_state() if static else None
     st = fn(in_dt, Q.ops._dt(c), scale_mode, layout, a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(),
             c.data_ptr(), c.stride(0), M, N, K, split, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if static:
+        # the property in the entry's name: neither the library's workspace nor the device's free memory moved
+        assert _memory_state() == before, (before, _memory_state())
     return st
 
 
@@ -86,3 +98,34 @@ def test_static_scratch_entry_refuses_what_does_not_fit():
     torch.cuda.synchronize()
     assert bool(torch.all(c == 3))                     # nothing was launched
     assert b"static scratch" in L.load_library().qgemm_status_string(10)
+    # the room for transposed operands counts too: reference layout through the transposes, A^T + B^T = 40 MiB
+    say("no-alloc entry: too large, transposed operands")
+    M, N, K = 4096, 6144, 4096
+    a = torch.zeros((K, M), dtype=torch.uint8, device="cuda")
+    b = torch.zeros((K, N), dtype=torch.uint8, device="cuda")
+    sa = torch.ones((K // 128, M), dtype=torch.float32, device="cuda")
+    sb = torch.ones((K // 128, N // 128), dtype=torch.float32, device="cuda")
+    cb = torch.full((M, N), 3.0, dtype=torch.bfloat16, device="cuda")
+    Q.set_option("kmajor", 0)
+    try:
+        assert _call(True, Q.DT_F8E4M3, Q.SCALE_BLOCK128, Q.LAYOUT_REFERENCE, a, b, sa, sb, cb, M, N, K, 1) == 10
+    finally:
+        Q.set_option("kmajor", 1)
+    torch.cuda.synchronize()
+    assert bool(torch.all(cb == 3.0))
+    # ... and the room for a transposed a_scale: 131072 rows x 72 K blocks of floats = 36 MiB
+    say("no-alloc entry: too large, transposed a_scale")
+    M, N, K = 131072, 128, 72 * 128 + 128
+    KB = K // 128                                      # odd: the kernels want a_scale rows-contiguous, through a copy
+    a = torch.zeros((M, K), dtype=torch.uint8, device="cuda")
+    b = torch.zeros((N, K), dtype=torch.uint8, device="cuda")
+    sa = torch.ones((M, KB), dtype=torch.float32, device="cuda")
+    sb = torch.ones((1, KB), dtype=torch.float32, device="cuda")
+    cb = torch.full((M, N), 3.0, dtype=torch.bfloat16, device="cuda")
+    Q.force_config("256x256_w2x4_solo8")
+    try:
+        assert _call(True, Q.DT_F8E4M3, Q.SCALE_BLOCK128, Q.LAYOUT_K_CONTIGUOUS, a, b, sa, sb, cb, M, N, K, 1) == 10
+    finally:
+        Q.force_config(None)
+    torch.cuda.synchronize()
+    assert bool(torch.all(cb == 3.0))
