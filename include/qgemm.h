@@ -123,7 +123,8 @@ int qgemm_scaled_gemm_static(int in_dtype, int out_dtype, int scale_mode, int la
  * device, through an event) for the previous user on another stream.  While a stream is being captured into a
  * graph the library neither allocates nor touches that event: a call that would have to grow the block returns
  * QGEMM_ERR_ALLOC, and replays of graphs that use the workspace must not overlap other users of it.
- * qgemm_reserve_workspace makes the block at least `bytes` large ahead of time; qgemm_workspace_info reports
+ * qgemm_reserve_workspace makes the block at least `bytes` large ahead of time (it allocates: call it before a
+ * capture begins, never during one; a block that has to grow at least doubles); qgemm_workspace_info reports
  * its address and size (NULL / 0 before first use). */
 int qgemm_reserve_workspace(size_t bytes);
 int qgemm_workspace_info(void **base, size_t *bytes);
@@ -159,10 +160,24 @@ int qgemm_quantize(int in_dtype, int out_dtype, int mode, const void *x, size_t 
 int qgemm_tile_map(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n, uint32_t group_m, uint32_t *tile_m,
                    uint32_t *tile_n);
 
-/* Tuning / diagnostics (no reference counterpart).
- * qgemm_set_option("force_config", i) pins tile configuration i (-1 = heuristic);
+/* Tuning / diagnostics (no reference counterpart: the reference picks its tile at compile time,
+ * src/include/gemm_config.h:30-36).
+ * qgemm_set_option(key, value): "force_split" (K slices, 0 = heuristic), "group_m", "kmajor", "stagger", "k_rot",
+ *   "as_groups", "row_split"; "force_config" accepts only -1 (back to the heuristic).
+ *   "k_rot": with at most 256 rows the workgroups of column tile i start their K loops 3 i steps in and wrap round
+ *   (memory channels), so the order of an fp32 sum depends on the column tile: results are the same from run to
+ *   run, but equal rows of A against equal columns of B at different column positions may differ in the last bits.
+ *   k_rot = 0 makes every workgroup start at K step 0 (position-independent sums); -1 restores the default.
+ * qgemm_force_config(name) pins the row `name` of the variant tables for every following GEMM call (NULL or "":
+ *   back to the heuristic).  Rows are addressed by name only; a call whose family has no row of that name returns
+ *   QGEMM_ERR_UNSUPPORTED, a name no family has is QGEMM_ERR_INVALID_ARG here.
+ * qgemm_variant_count / qgemm_variant_name enumerate the rows of the family that serves (in_dtype, scale_mode,
+ *   k_major) -- arguments as for qgemm_plan -- so that callers never depend on the order of a table.
  * qgemm_last_config writes the name of the kernel variant the last GEMM call chose. */
 int qgemm_set_option(const char *key, long value);
+int qgemm_force_config(const char *name);
+int qgemm_variant_count(int in_dtype, int scale_mode, int k_major);
+int qgemm_variant_name(int in_dtype, int scale_mode, int k_major, int index, char *buf, size_t buflen);
 int qgemm_last_config(char *buf, size_t buflen);
 
 /* Which kernel configuration the library would run for a problem with dense, 16-byte aligned operands: the name

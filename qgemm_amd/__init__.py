@@ -10,5 +10,5 @@ from .ops import (  # noqa: F401
     LAYOUT_K_CONTIGUOUS, LAYOUT_REFERENCE, QUANT_BLOCK_128x128, QUANT_BLOCK_1x128, QUANT_PER_MATRIX,
     SCALE_BLOCK128, SCALE_PER_MATRIX,
     bf16_mm, fp8_mm, gemm, int8_mm, last_config, matrix_transpose, plan, quantize, scaled_gemm, selftest_layouts,
-    set_option, tile_map,
+    force_config, set_option, tile_map, variant_names,
 )

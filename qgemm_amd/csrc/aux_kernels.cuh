@@ -314,13 +314,11 @@ __global__ void __launch_bounds__(256) splitk_reduce4_kernel(const ReduceArgs p,
         else
             for (int e = 0; e < 4; ++e) dst[e] = v[e];
     } else {
-        unsigned short h[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) h[e] = p.out_dtype == QGEMM_DT_BF16 ? f32_to_bf16_bits(v[e]) : f32_to_f16_bits(v[e]);
+        const v2i h = p.out_dtype == QGEMM_DT_BF16 ? pack4_bf16(v[0], v[1], v[2], v[3]) : pack4_f16(v[0], v[1], v[2], v[3]);
         unsigned short *dst = (unsigned short *)p.C + idx;
-        if (c_vec) *(us4 *)dst = us4{h[0], h[1], h[2], h[3]};
+        if (c_vec) *(v2i *)dst = h;
         else
-            for (int e = 0; e < 4; ++e) dst[e] = h[e];
+            for (int e = 0; e < 4; ++e) dst[e] = pack4_elem(h, e);
     }
 }
 

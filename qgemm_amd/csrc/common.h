@@ -42,6 +42,24 @@ __device__ inline unsigned short f32_to_f16_bits(float f) {
     _Float16 h = (_Float16)f;
     return __builtin_bit_cast(unsigned short, h);
 }
+// Four floats -> four bf16 / fp16 values in 8 bytes, element 0 in the low half of component 0.  Two elements per
+// v_cvt_pk_*: half the instructions of four scalar conversions, and no packing step afterwards.  (The packing the
+// compiler picks for two 16-bit scalars, v_pack_b32_f16, treats its inputs as fp16 numbers and quiets what looks
+// like a signalling NaN: a bf16 pattern 0x7c01 .. 0x7dff, a finite value of 2^121 and more, came out with bit 9
+// set.  The vector conversions never hold a lone 16-bit value in a register.)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ inline v2i pack4_bf16(float a, float b, float c, float d) {
+    return v2i{__builtin_bit_cast(int, __builtin_convertvector(f32x2_t{a, b}, bf16x2_t)),
+               __builtin_bit_cast(int, __builtin_convertvector(f32x2_t{c, d}, bf16x2_t))};
+}
+__device__ inline v2i pack4_f16(float a, float b, float c, float d) {
+    return v2i{__builtin_bit_cast(int, __builtin_convertvector(f32x2_t{a, b}, f16x2_t)),
+               __builtin_bit_cast(int, __builtin_convertvector(f32x2_t{c, d}, f16x2_t))};
+}
+// element e (0 .. 3) of such a pack
+__device__ inline unsigned short pack4_elem(v2i p, int e) { return (unsigned short)((unsigned)p[e >> 1] >> ((e & 1) * 16)); }
 
 // Linear workgroup id -> (tile_m, tile_n).
 // Step 1 (XCD remap): the dispatcher deals workgroups to the 8 XCDs round

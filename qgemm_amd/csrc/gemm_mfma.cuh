@@ -73,36 +73,20 @@ struct GemmArgs {
     unsigned long long *dbg_cycles;   // measurement builds only (QGEMM_STAMP): time stamps per wave
 };
 
-// How a stage travels from global memory to LDS.
-//   LOAD_DMA   buffer_load_dwordx4 ... lds: no VGPR staging, the wave only waits on vmcnt
-//   LOAD_VGPR  buffer_load_dwordx4 into registers during the MFMAs of the previous
-//              tile, ds_write_b128 afterwards; same addresses, same LDS layout
-enum Loader : int { LOAD_DMA = 0, LOAD_VGPR = 1 };
-
 // How the K loop is scheduled.
 //   PIPE_SIMPLE    every wave: wait for tile k, barrier, start tile k+1, read fragments, MFMA.
-//   PIPE_PINGPONG  8 waves = 2 per SIMD.  Waves 0-3 and waves 4-7 run the same loop half a K
-//                  step apart: while one wave of a SIMD issues the MFMAs of tile k from
-//                  registers, its partner reads the fragments of its next tile from LDS and
-//                  starts the next global -> LDS copy.  The matrix core of every SIMD always
-//                  has one wave feeding it; barriers fall between the phases.
 //   PIPE_SOLO      4 waves = 1 per SIMD, each with a 128 x 128 wave tile (64 accumulator tiles).  A
 //                  fragments are streamed two rows of MFMAs ahead, B fragments of step k+1 replace
 //                  those of step k as they die in its last two rows, copies ride between the MFMAs:
-//                  a third fewer LDS reads per MFMA than the ping-pong pipeline and one barrier
-//                  per K step.  A triple-buffered, B double-buffered in LDS (same 160 KiB).
+//                  few LDS reads per MFMA and one barrier per K step.  A triple-buffered, B
+//                  double-buffered in LDS (160 KiB for 256 x 256).
 //                  With 8 waves (128 x 64 wave tiles) the same schedule runs two waves per SIMD and
 //                  keeps the accumulators in vector registers, which the block-scale fold needs.
-enum Pipe : int { PIPE_SIMPLE = 0, PIPE_PINGPONG = 1, PIPE_SOLO = 2 };
+// Global -> LDS always goes through buffer_load_dwordx4 ... lds: no VGPR staging, the wave only waits on vmcnt.
+enum Pipe : int { PIPE_SIMPLE = 0, PIPE_SOLO = 2 };
 
-// TAIL_ (ping-pong): number of B-fragment columns of MFMAs a wave still issues after the
-// barrier that ends its compute phase, so the hand-over to its partner is hidden.
-// A3_   (ping-pong): A gets three LDS buffers and B two (exactly 160 KiB for 256 x 256):
-// the A copy of tile k+2 is started two K steps ahead and only the B half of a tile has to
-// land within one step.
-template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int LOADER_ = LOAD_DMA,
-          int PIPE_ = PIPE_SIMPLE, int TAIL_ = 0, bool A3_ = false, int KMAJ_ = 0, int STAGES_ = 0, int KGROUPS_ = 1,
-          bool ASK_ = false, bool COPYW_ = false>
+template <int ARITH_, bool BLOCK_SCALE_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, int PIPE_ = PIPE_SIMPLE,
+          int KMAJ_ = 0, int STAGES_ = 0, int KGROUPS_ = 1, bool ASK_ = false, bool COPYW_ = false>
 struct GemmCfg {
     // COPYW (solo pipeline, four computing waves with 128 x 64 wave tiles on a 256 x 128 tile): four more waves issue
     // every copy of the K loop, at the places the schedule has them; the computing waves, one per SIMD, issue fragment
@@ -114,7 +98,7 @@ struct GemmCfg {
     // arrangement of QGEMM_LAYOUT_K_CONTIGUOUS, instead of rows contiguous, a_scale[m + kb * as_ks].  A compile-time
     // choice: as a branch inside the K loop it cost the 8-wave kernel 758 spilled registers.
     static constexpr bool ASK = ASK_;
-    // The simple and ping-pong pipelines load one scale per lane and K step at a_scale[m * as_ms + kb * as_ks] with
+    // The simple pipeline loads one scale per lane and K step at a_scale[m * as_ms + kb * as_ks] with
     // whatever strides they are given: rows-contiguous scales are one 256-byte request per 64 rows, K-contiguous
     // ones 64 requests, which these tiles (a step of several hundred cycles per wave) can afford and which saves the
     // launch that would copy the scales into the other order.
@@ -133,10 +117,8 @@ struct GemmCfg {
     static constexpr bool KMA = (KMAJ_ & 1) != 0, KMB = (KMAJ_ & 2) != 0;
     static constexpr int ES = (ARITH_ == AR_BF16 || ARITH_ == AR_F16) ? 2 : 1;   // operand element bytes
     static constexpr int KE = 128 / ES;                                          // K elements per step
-    static constexpr int LOADER = LOADER_;
     static constexpr int PIPE = PIPE_;
-    static constexpr int TAIL = TAIL_;
-    static constexpr bool A3 = A3_;
+    static constexpr bool A3 = PIPE_ == PIPE_SOLO;      // solo: three A buffers and two B buffers instead of whole stages
     static constexpr int ARITH = ARITH_;
     static constexpr bool BLOCK_SCALE = BLOCK_SCALE_;
     static constexpr int BM = BM_, BN = BN_, BKB = 128;         // BKB: bytes of K per step
@@ -152,7 +134,7 @@ struct GemmCfg {
     static constexpr int LPT = NLOAD / NW;                      // ... per wave
     static constexpr int A_BYTES = RBA * 2048, B_BYTES = RBB * 2048;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int LPT_A = RBA * 2 / NW;                  // A load instructions per wave (ping-pong)
+    static constexpr int LPT_A = RBA * 2 / NW;                  // A load instructions per wave
     // simple pipeline with the DMA loader: as many stages in flight as LDS and the 6-bit vmcnt allow (at most
     // 8).  A workgroup that streams a narrow strip of B (skinny M) otherwise waits one full memory round trip
     // per K step.  The block-scale form keeps two (its scale loads share vmcnt with the copies), except with K
@@ -161,7 +143,7 @@ struct GemmCfg {
     // Only for the small tiles: a 128 x 128 tile with two stages leaves room for two workgroups per CU, which is
     // worth more to a compute-bound shape than deeper prefetch.
     static constexpr int NSTAGE = STAGES_ > 0 ? STAGES_
-                                  : (PIPE != PIPE_SIMPLE || LOADER != LOAD_DMA || BLOCK_SCALE || BM * BN > 64 * 128 || KMAJ_ != 0) ? 2
+                                  : (PIPE != PIPE_SIMPLE || BLOCK_SCALE || BM * BN > 64 * 128 || KMAJ_ != 0) ? 2
                                   : (NSTAGE_FIT < NSTAGE_CNT ? (NSTAGE_FIT < 8 ? NSTAGE_FIT : 8)
                                                              : (NSTAGE_CNT < 8 ? NSTAGE_CNT : 8));
     // Block scales with K groups: the a_scale values of a stage (one float per tile row, at most 128) travel to LDS
@@ -172,27 +154,24 @@ struct GemmCfg {
     static constexpr int SCALE_LDS = (BLOCK_SCALE_ && KGROUPS_ == 2) ? (NSTAGE * 512 > 64 * BM_ ? NSTAGE * 512 : 64 * BM_)
                                      : (BLOCK_SCALE_ && COPYW_ && ASK_) ? 64 * BM_ : 0;
     static constexpr int LDS_BYTES = (A3 ? 3 * A_BYTES + 2 * B_BYTES : NSTAGE * STAGE_BYTES) + SCALE_LDS;
-    static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA && (!BLOCK_SCALE || KGROUPS_ == 2) &&
+    static_assert(STAGES_ == 0 || (PIPE == PIPE_SIMPLE && (!BLOCK_SCALE || KGROUPS_ == 2) &&
                                    (KMAJ_ == 0 || KGROUPS_ == 2) && STAGES_ >= 2 && STAGES_ <= NSTAGE_FIT && STAGES_ <= NSTAGE_CNT),
-                  "explicit stage count: simple pipeline, DMA loader, within LDS and the 6-bit counter");
-    static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && PIPE == PIPE_SIMPLE && LOADER == LOAD_DMA &&
+                  "explicit stage count: simple pipeline, within LDS and the 6-bit counter");
+    static_assert(KGROUPS_ == 1 || (KGROUPS_ == 2 && PIPE == PIPE_SIMPLE &&
                                     NSTAGE >= 4 && (!BLOCK_SCALE_ || (BM_ <= 128 && BN_ <= 128))),
-                  "K groups: simple pipeline, DMA loader, at least four stages");
+                  "K groups: simple pipeline, at least four stages");
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
     static_assert(NLOAD % NW == 0, "load instructions must divide evenly over the waves");
     static_assert(!BLOCK_SCALE || ARITH == AR_F8, "block scales are defined for fp8 only");
     static_assert(!BLOCK_SCALE || (128 % WN == 0 || WN % 128 == 0), "wave tile must align with 128-wide scale blocks");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS is 160 KiB per CU");
-    static_assert(PIPE != PIPE_PINGPONG || (NW == 8 && LOADER == LOAD_DMA), "ping-pong needs 8 waves and the DMA loader");
-    static_assert(PIPE != PIPE_SOLO || ((NW == 4 || NW == 8) && LOADER == LOAD_DMA && A3 && TN >= 4 &&
+    static_assert(PIPE != PIPE_SOLO || ((NW == 4 || NW == 8) && TN >= 4 &&
                                         ((TM % 4 == 0 && TM >= 8) || (TM == 6 && NW == 8))),
-                  "solo: 4 or 8 waves, DMA loader, A triple-buffered, at least 8 rows (8 waves: or 6) of at least 4 MFMAs per step");
+                  "solo: 4 or 8 waves, at least 8 rows (8 waves: or 6) of at least 4 MFMAs per step");
     static_assert(!COPYW_ || (PIPE_ == PIPE_SOLO && WAVES_M_ * WAVES_N_ == 4 && KGROUPS_ == 1), "copying waves beside four computing waves: solo pipeline");
     static_assert(PIPE != PIPE_SOLO || !BLOCK_SCALE || NW == 8 || COPYW_,
                   "solo with block scales: the accumulators have to live in the 256 vector registers of a wave");
     static_assert(PIPE == PIPE_SIMPLE || (RBA * 2) % NW == 0, "A loads must divide evenly over the waves");
-    static_assert(PIPE != PIPE_SIMPLE || (TAIL == 0 && !A3), "TAIL and A3 belong to the pipelined variants");
-    static_assert(TAIL >= 0 && TAIL < TN, "TAIL counts B-fragment columns");
     static_assert(KMAJ == 0 || NW % 4 == 0, "K-major tiles: the swizzle of a copy must not depend on the instruction");
     static_assert((!KMA || (BM * ES) % 128 == 0) && (!KMB || (BN * ES) % 128 == 0),
                   "K-major tiles are made of whole 128-byte panels");
@@ -404,7 +383,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         return blk * 16 * ld + (uint32_t)kt * C::BKB;
     };
 
-    auto issue_stage = [&](int kt) {       // LOAD_DMA: global -> LDS
+    auto issue_stage = [&](int kt) {       // global -> LDS
         char *stage = smem + (kt % C::NSTAGE) * C::STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < C::LPT; ++i) {
@@ -416,25 +395,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         }
     };
 
-    v4i staged[C::LOADER == LOAD_VGPR ? C::LPT : 1];
-    auto fetch_stage = [&](int kt) {       // LOAD_VGPR: global -> registers
-#pragma unroll
-        for (int i = 0; i < C::LPT; ++i)
-            staged[i] = i < LPT_A0 ? __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a, load_soff(i, kt), 0)
-                                   : __builtin_amdgcn_raw_buffer_load_b128(rb, voff_b, load_soff(i, kt), 0);
-    };
-    auto commit_stage = [&](int kt) {      // LOAD_VGPR: registers -> LDS, where the DMA would have put them
-        char *stage = smem + (kt & 1) * C::STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < C::LPT; ++i) *(v4i *)(stage + (wave + i * C::NW) * 1024 + lane * 16) = staged[i];
-    };
-
     // ---- block scales (fp8 only): a_scale per row of each A fragment, b_scale per 128 columns.
     // a_scale is read with the rows contiguous (as_ms == 1: a_scale[m + kb*as_ks], the host guarantees it):
     // lane l fetches the scale of wave-tile row l (and l + 64), one 256-byte request per 64 rows, through a
     // buffer load (rows past M read as 0 or as some other finite scale; they only meet zero operands).  A
     // step later every lane picks the row of each of its A fragments (row l & 15 of row block a) out of
-    // those registers: with ds_bpermute in the simple and ping-pong pipelines, with lane swaps on the vector
+    // those registers: with ds_bpermute in the simple pipeline, with lane swaps on the vector
     // ALU in the solo pipeline.  One load per lane and fragment instead (16 distinct rows per instruction,
     // every row a request of its own) keeps the texture addresser busy for longer than the MFMAs of the
     // step take.
@@ -528,25 +494,9 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // ---- K loop
     QGEMM_STAMP(1);
     if constexpr (C::PIPE != PIPE_SIMPLE) {
-        // (ping-pong) Waves 4-7 ("late" group) run one phase behind waves 0-3 ("early" group).  Phases:
-        //   memory : ds_read all fragments of tile kt into registers
-        //   compute: MFMAs of tile kt, operands all in registers
-        // so whenever one wave of a SIMD is in its compute phase its partner is in its memory
-        // phase, and every phase boundary is one workgroup barrier ("slot" 2kt: early group reads
-        // tile kt, late group computes tile kt-1; slot 2kt+1: the other way round).
-        //
-        // Global -> LDS copies are issued one at a time between the ds_reads / MFMAs of a
-        // phase (a burst in front of the MFMAs would hold them back while the texture
-        // addresser works through the queue).  With A3: every wave issues its share of B(kt+1)
-        // in slot 2kt and of A(kt+2) in slot 2kt+1, and waits with vmcnt(LPT_A) at the end of
-        // every odd slot: that leaves only the A copy just issued, which has two more slots to
-        // land, in flight.  Without A3 both A(kt+1) and B(kt+1) go out in slot 2kt.
         // A buffer is first read one barrier after the wait of its last copier, and is first
         // overwritten one barrier after the lgkmcnt(0) of its last reader.
-        //
-        // The loop exists four times (early / late group, with / without the end-of-K guards)
-        // so that the steady state has no branches between the MFMAs.
-        constexpr int NA_BUF = C::A3 ? 3 : 2;
+        constexpr int NA_BUF = 3;
         constexpr int B_BASE = NA_BUF * C::A_BYTES;
         constexpr int LPT_A = C::LPT_A, LPT_B = C::LPT - C::LPT_A;
         // instruction i < LPT_A of this wave belongs to A, the rest to B (RBA*2 % NW == 0)
@@ -972,174 +922,17 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // before the epilogue reads the accumulators
                 if constexpr (PINNED) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
             }
-        } else {
-            // The copies of one slot as a numbered list 0 .. n-1, so a phase can issue them one by one.
-            //   even slot 2kt  : A3 ? B(kt+1)            : A(kt+1) then B(kt+1)
-            //   odd slot 2kt+1 : A3 ? A(kt+2) -> a_wr     : nothing
-            constexpr int N_EVEN = C::A3 ? LPT_B : C::LPT, N_ODD = C::A3 ? LPT_A : 0;
-            int a_wr = C::A3 ? 2 : 1;           // buffer the next A copy of this wave goes to
-            int a_rd = 0;                       // buffer holding A of the tile being read
-            // kt: tile the early group reads in this slot; guard: check the end of K
-            auto issue_even = [&](int j, int kt, bool guard) {
-                if (guard && kt + 1 >= nk) return;
-                if constexpr (C::A3) issue_b1(LPT_A + j, kt + 1);
-                else if (j < LPT_A) issue_a1(j, kt + 1, a_wr);
-                else issue_b1(j, kt + 1);
-            };
-            auto issue_odd = [&](int j, int kt, bool guard) {
-                if constexpr (C::A3) {
-                    if (guard && kt + 2 >= nk) return;
-                    issue_a1(j, kt + 2, a_wr);
-                }
-            };
-            v4i fa[C::TM][2], fb[C::TN][2];
-            constexpr int COLS_COPY = C::TN - C::TAIL;    // copies that can ride between the MFMA columns
-
-            // one K step of one wave.  LATE / GUARD are std::integral_constant<bool>.
-            auto step = [&](int kt, auto late_tag, auto guard_tag) {
-                constexpr bool LATE = decltype(late_tag)::value, GUARD = decltype(guard_tag)::value;
-                // ---- memory phase (early: slot 2kt, even; late: slot 2kt+1, odd)
-                if constexpr (C::BLOCK_SCALE) {
-                    expand_scales();
-                    if (!GUARD || kt + 1 < nk) fetch_scales(kt + 1);
-                }
-                const char *sa_ = smem + a_rd * C::A_BYTES;
-                const char *sb_ = smem + B_BASE + (kt & 1) * C::B_BYTES - C::A_BYTES;   // frag_b adds RBA row blocks
-                constexpr int n_m = LATE ? N_ODD : N_EVEN;     // copies of this wave in this phase
-    #pragma unroll
-                for (int a = 0; a < C::TM; ++a) {
-                    if (a < n_m) {
-                        if constexpr (LATE) issue_odd(a, kt, GUARD);
-                        else issue_even(a, kt, GUARD);
-                    }
-                    fa[a][0] = frag_a(sa_, a, 0);
-                    fa[a][1] = frag_a(sa_, a, 1);
-                }
-    #pragma unroll
-                for (int b = 0; b < C::TN; ++b) {
-                    if (C::TM + b < n_m) {
-                        if constexpr (LATE) issue_odd(C::TM + b, kt, GUARD);
-                        else issue_even(C::TM + b, kt, GUARD);
-                    }
-                    fb[b][0] = frag_b(sb_, b, 0);
-                    fb[b][1] = frag_b(sb_, b, 1);
-                }
-                if constexpr (LATE ? (N_ODD > 0) : !C::A3) a_wr = next_buf(a_wr);
-                a_rd = next_buf(a_rd);
-                __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());   // reads done before the buffers may be refilled
-                auto wait_copies = [&]() {   // end of an odd slot: all copies landed but (A3) the A copy just issued
-                    __builtin_amdgcn_sched_barrier(0);   // stays behind the MFMAs of the phase
-                    if (C::A3 && (!GUARD || kt + 2 < nk)) __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
-                    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-                };
-                if constexpr (LATE) wait_copies();
-                phase_barrier();
-                // ---- compute phase (early: slot 2kt+1, odd; late: slot 2kt+2, even)
-                constexpr int n_c = LATE ? N_EVEN : N_ODD;
-                const int kt_slot = LATE ? kt + 1 : kt;
-    #pragma unroll
-                for (int j = COLS_COPY; j < n_c; ++j) {        // copies that do not fit between the columns
-                    if constexpr (LATE) issue_even(j, kt_slot, GUARD);
-                    else issue_odd(j, kt_slot, GUARD);
-                }
-                // block scales: one factor per A-fragment row block and 128-column block for this K step
-                float sc[C::BLOCK_SCALE ? C::TM : 1][NBS];
-                if constexpr (C::BLOCK_SCALE) {
-    #pragma unroll
-                    for (int a = 0; a < C::TM; ++a)
-    #pragma unroll
-                        for (int j = 0; j < NBS; ++j) sc[a][j] = as_cur[a] * bs_cur[j];
-                }
-                auto mfma_cols = [&](int b0, int b1, int ncopy) {
-                    if constexpr (C::BLOCK_SCALE) {
-                        // partial product of this 128-wide K block into a fresh accumulator, folded into
-                        // the running sum with one FMA per element (hip_mix_gemm_kernel.cpp:231-244), one
-                        // MFMA behind so the FMAs of tile i run under the MFMA of tile i+1
-                        v4f part[2];
-    #pragma unroll
-                        for (int i = b0 * C::TM; i <= b1 * C::TM; ++i) {
-                            const int a = i % C::TM, b = i / C::TM;
-                            if (i < b1 * C::TM) {
-                                if (a == 0 && b < ncopy) {
-                                    if constexpr (LATE) issue_even(b, kt_slot, GUARD);
-                                    else issue_odd(b, kt_slot, GUARD);
-                                }
-                                part[i & 1] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
-                            }
-                            __builtin_amdgcn_sched_barrier(0);   // MFMA i first, the FMAs of tile i-1 under it
-                            if (i > b0 * C::TM) {
-                                const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
-                                const float f = sc[pa][(pb * 16) / 128];
-    #pragma unroll
-                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f;
-                            }
-                            __builtin_amdgcn_sched_barrier(0);
-                        }
-                        return;
-                    }
-    #pragma unroll
-                    for (int b = b0; b < b1; ++b) {
-                        if (b < ncopy) {              // one copy in front of each of the first columns
-                            if constexpr (LATE) issue_even(b, kt_slot, GUARD);
-                            else issue_odd(b, kt_slot, GUARD);
-                            __builtin_amdgcn_sched_barrier(0);
-                        }
-    #pragma unroll
-                        for (int a = 0; a < C::TM; ++a)
-                            acc[a][b] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], acc[a][b]);
-                    }
-                };
-                mfma_cols(0, C::TN - C::TAIL, n_c < COLS_COPY ? n_c : COLS_COPY);
-                if constexpr (LATE ? !C::A3 : (N_ODD > 0)) a_wr = next_buf(a_wr);
-                if constexpr (!LATE) wait_copies();
-                if (!LATE || !GUARD || kt + 1 < nk) phase_barrier();
-                mfma_cols(C::TN - C::TAIL, C::TN, 0);
-            };
-
-            if (nk > 0) {
-                fetch_scales(0);
-    #pragma unroll
-                for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
-    #pragma unroll
-                for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 0);
-                if (C::A3 && nk > 1) {
-    #pragma unroll
-                    for (int i = 0; i < LPT_A; ++i) issue_a1(i, 1, 1);
-                    __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
-                } else {
-                    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-                }
-                phase_barrier();
-            }
-            typedef std::integral_constant<bool, true> yes_t;
-            typedef std::integral_constant<bool, false> no_t;
-            const int nk_fast = nk > 3 ? nk - 3 : 0;    // steps that cannot touch the end of K
-            if (wave >= C::NW / 2) {
-                if (nk > 0) {                   // slot 0 of the late group: only its copies
-    #pragma unroll
-                    for (int j = 0; j < N_EVEN; ++j) issue_even(j, 0, true);
-                    if (!C::A3) a_wr = next_buf(a_wr);
-                    phase_barrier();
-                }
-                int kt = 0;
-                for (; kt < nk_fast; ++kt) step(kt, yes_t{}, no_t{});
-                for (; kt < nk; ++kt) step(kt, yes_t{}, yes_t{});
-            } else {
-                int kt = 0;
-                for (; kt < nk_fast; ++kt) step(kt, no_t{}, no_t{});
-                for (; kt < nk; ++kt) step(kt, no_t{}, yes_t{});
-            }
         }
     } else {
         constexpr int NS = C::NSTAGE;
-        // The barrier of a step.  With the DMA loader it is the bare s_barrier behind the wave's own wait for its
+        // The barrier of a step: the bare s_barrier behind the wave's own wait for its
         // copies (counted, see below): __syncthreads() carries a fence that the compiler turns into "wait for every
         // copy in flight", which empties the ring at every step and leaves the stages issued ahead no time to land
         // under the MFMAs.  Fragment reads are complete before their MFMAs issue, so a wave that reaches the barrier
-        // has left the buffers the next copies overwrite.  (Register staging writes LDS with ds_write and needs the
-        // full barrier; so do the K-major tiles, whose transposing reads the compiler orders behind all copies.)
+        // has left the buffers the next copies overwrite.  (The K-major tiles, whose transposing reads the compiler
+        // orders behind all copies, take the full barrier.)
         auto ring_barrier = [&]() {
-            if constexpr (C::LOADER == LOAD_DMA && C::KMAJ == 0) phase_barrier();
+            if constexpr (C::KMAJ == 0) phase_barrier();
             else __syncthreads();
         };
         // Small tiles with a deep ring (NS >= 4): two K steps per barrier.  A workgroup of these is alone or nearly
@@ -1147,7 +940,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
         // 0.25 - 0.36 us; taking the steps in pairs pays the barrier and the LDS latency once for two.  Before turn
         // kt (even) stages 0 .. kt+NS-3 have been issued; stages kt and kt+1 are waited for, everybody leaves the
         // buffers of kt-2 and kt-1, and stages kt+NS-2 and kt+NS-1 are issued into them.
-        constexpr bool PAIRS = NS >= 4 && C::LOADER == LOAD_DMA && !C::BLOCK_SCALE && C::KMAJ == 0 && C::BM * C::BN <= 64 * 128 &&
+        constexpr bool PAIRS = NS >= 4 && !C::BLOCK_SCALE && C::KMAJ == 0 && C::BM * C::BN <= 64 * 128 &&
                                C::KG == 1;
         if constexpr (C::KG == 2) {
             // Two sets of waves half a turn apart, and four waves that copy.  Phase s opens with a barrier; behind it
@@ -1365,33 +1158,23 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             }
         } else {
         if (nk > 0) {
-            if constexpr (C::LOADER == LOAD_DMA) {
 #pragma unroll
-                for (int j = 0; j < NS - 1; ++j)
-                    if (j < nk) issue_stage(j);
-            } else {
-                fetch_stage(0);
-                commit_stage(0);
-            }
+            for (int j = 0; j < NS - 1; ++j)
+                if (j < nk) issue_stage(j);
             fetch_scales(0);
         }
         for (int kt = 0; kt < nk; ++kt) {
-            if constexpr (C::LOADER == LOAD_DMA) {
-                // this wave's part of tile kt has landed: everything but the NS-2 stages issued after it
-                // (near the end of K fewer are in flight: wait for all)
-                if (NS > 2 && kt + NS - 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * C::LPT));
-                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-            }
+            // this wave's part of tile kt has landed: everything but the NS-2 stages issued after it
+            // (near the end of K fewer are in flight: wait for all)
+            if (NS > 2 && kt + NS - 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * C::LPT));
+            else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
             ring_barrier();                                  // ... and everybody else's; tile kt-1 is fully consumed
             expand_scales();
             auto next_stage = [&]() {                        // into the buffer tile kt-1 has just left
-                if (kt + NS - 1 < nk) {
-                    if constexpr (C::LOADER == LOAD_DMA) issue_stage(kt + NS - 1);
-                    else fetch_stage(kt + 1);
-                }
+                if (kt + NS - 1 < nk) issue_stage(kt + NS - 1);
             };
             // K-major tiles: all fragment reads of the step first, the copies behind them (see GemmCfg)
-            constexpr bool READS_FIRST = C::KMAJ != 0 && C::LOADER == LOAD_DMA;
+            constexpr bool READS_FIRST = C::KMAJ != 0;
             if constexpr (!READS_FIRST) next_stage();
             if (kt + 1 < nk) fetch_scales(kt + 1);
             const char *stage = smem + (kt % NS) * C::STAGE_BYTES;
@@ -1442,10 +1225,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 }
             }
             if constexpr (C::BLOCK_SCALE) fold_tile(C::TM * C::TN - 1);
-            if constexpr (C::LOADER == LOAD_VGPR) {
-                // the other stage was last read in iteration kt-1, which every wave left before this one began
-                if (kt + 1 < nk) commit_stage(kt + 1);
-            }
         }
         }
     }
@@ -1559,13 +1338,11 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 } else if (DT == QGEMM_DT_BF16) {
 #pragma unroll
                     for (int b = 0; b < C::TN; ++b)
-                        *(us4 *)(wr + b * 16 * 2) = us4{f32_to_bf16_bits(v[b][0]), f32_to_bf16_bits(v[b][1]),
-                                                        f32_to_bf16_bits(v[b][2]), f32_to_bf16_bits(v[b][3])};
+                        *(v2i *)(wr + b * 16 * 2) = pack4_bf16(v[b][0], v[b][1], v[b][2], v[b][3]);
                 } else {
 #pragma unroll
                     for (int b = 0; b < C::TN; ++b)
-                        *(us4 *)(wr + b * 16 * 2) = us4{f32_to_f16_bits(v[b][0]), f32_to_f16_bits(v[b][1]),
-                                                        f32_to_f16_bits(v[b][2]), f32_to_f16_bits(v[b][3])};
+                        *(v2i *)(wr + b * 16 * 2) = pack4_f16(v[b][0], v[b][1], v[b][2], v[b][3]);
                 }
             }
         };
@@ -1637,15 +1414,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     for (int r = 0; r < 4; ++r)
                         if (n + r < p.N) dst[r] = v[r];
             } else {
-                unsigned short h[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    h[r] = p.out_dtype == QGEMM_DT_BF16 ? f32_to_bf16_bits(v[r]) : f32_to_f16_bits(v[r]);
+                const v2i h = p.out_dtype == QGEMM_DT_BF16 ? pack4_bf16(v[0], v[1], v[2], v[3]) : pack4_f16(v[0], v[1], v[2], v[3]);
                 unsigned short *dst = (unsigned short *)Cz + idx;
-                if (full) *(us4 *)dst = us4{h[0], h[1], h[2], h[3]};
+                if (full) *(v2i *)dst = h;
                 else
                     for (int r = 0; r < 4; ++r)
-                        if (n + r < p.N) dst[r] = h[r];
+                        if (n + r < p.N) dst[r] = pack4_elem(h, r);
             }
         }
     }

@@ -385,15 +385,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
                 for (int r = 0; r < 4; ++r)
                     if (n + r < p.N) dst[r] = v[r];
         } else {
-            unsigned short h[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                h[r] = p.out_dtype == QGEMM_DT_BF16 ? f32_to_bf16_bits(v[r]) : f32_to_f16_bits(v[r]);
+            const v2i h = p.out_dtype == QGEMM_DT_BF16 ? pack4_bf16(v[0], v[1], v[2], v[3]) : pack4_f16(v[0], v[1], v[2], v[3]);
             unsigned short *dst = (unsigned short *)Cz + idx;
-            if (full) *(us4 *)dst = us4{h[0], h[1], h[2], h[3]};
+            if (full) *(v2i *)dst = h;
             else
                 for (int r = 0; r < 4; ++r)
-                    if (n + r < p.N) dst[r] = h[r];
+                    if (n + r < p.N) dst[r] = pack4_elem(h, r);
         }
     }
     QGEMM_STAMP(5);

@@ -54,7 +54,7 @@ struct Context {
     bool ws_used_by_call = false;              // the running entry asked for the workspace
     bool static_call = false;                  // the running entry takes its workspace from the static scratch
     void *static_ptr[kMaxDevices] = {};        // device address of `scratch`, per device
-    long force_config = -1;     // index into the variant table, -1 = heuristic
+    std::string force_config;   // name of a row of the variant tables, empty = heuristic (qgemm_force_config)
     long force_split = 0;       // 0 = heuristic
     long force_group_m = 0;     // 0 = default
 #if QGEMM_DEBUG_BUILD
@@ -87,13 +87,15 @@ int ensure_init_locked() {
     HIP_TRY(hipGetDevice(&dev));
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, dev));
-    void *scratch_dev = nullptr;               // address of the static scratch on this device, kept for later
-    int sst = static_scratch_locked(&scratch_dev);
-    if (sst != QGEMM_OK) return sst;
+    // The address of the static scratch on this device is looked up here, once, so that qgemm_scaled_gemm_static
+    // finds it without a runtime call of its own; if the lookup fails only that entry is affected (it tries again
+    // and reports the failure), every other entry works without the scratch.
+    void *scratch_dev = nullptr;
+    (void)static_scratch_locked(&scratch_dev);
     g_ctx.device = dev;
     g_ctx.num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     // tuning knobs, also reachable through qgemm_set_option
-    if (const char *e = std::getenv("QGEMM_FORCE_CONFIG")) g_ctx.force_config = std::atol(e);
+    if (const char *e = std::getenv("QGEMM_FORCE_CONFIG")) g_ctx.force_config = e;
     if (const char *e = std::getenv("QGEMM_GROUP_M")) g_ctx.force_group_m = std::atol(e);
     g_ctx.ready = true;
     return QGEMM_OK;
@@ -192,6 +194,14 @@ const Variant *table_for(int arith, bool block, int kmaj, int *count) {
     }
     return nullptr;
 }
+
+// Row `name` of a table, -1 when the family has no such row.
+int row_by_name(const Variant *tab, int count, const std::string &name) {
+    for (int i = 0; tab && i < count; ++i)
+        if (name == tab[i].name) return i;
+    return -1;
+}
+bool forced() { return !g_ctx.force_config.empty(); }
 
 int arith_of(int in_dtype) {
     switch (in_dtype) {
@@ -455,8 +465,8 @@ bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes
     if (!mfma_shape_ok(q)) return false;
     int count = 0, count_km = 0;
     const Variant *tab = table_for(q.arith, q.block, 0, &count), *tab_km = table_for(q.arith, q.block, kmaj, &count_km);
-    if (!tab || !tab_km || count != count_km) return false;
-    if (g_ctx.force_config >= 0 && g_ctx.force_config < count) return true;    // forced rows exist in every family
+    if (!tab || !tab_km) return false;
+    if (forced()) return row_by_name(tab_km, count_km, g_ctx.force_config) >= 0;   // a forced row: as stored where the K-major family has it
     if (g_ctx.kmajor == 2) return true;                                        // measurements: as stored wherever possible
     const size_t ksteps = q.Kbytes / 128;
     const bool may_split = q.split_k == 0;
@@ -516,7 +526,7 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
     if (!tab) return QGEMM_ERR_UNSUPPORTED;
     uint32_t model_split = 0;
     int vi = choose_variant(tab, count, q.M, q.N, q.Kbytes / 128, q.block, q.kmaj, g_ctx.num_cus, q.split_k == 0, &model_split);
-    if (may_split_rows && vi >= 0 && g_ctx.force_config < 0 && g_ctx.force_split <= 0 && q.split_k == 0 && model_split <= 1 &&
+    if (may_split_rows && vi >= 0 && !forced() && g_ctx.force_split <= 0 && q.split_k == 0 && model_split <= 1 &&
         q.M > 128 && q.kmaj == 0) {
         uint32_t ns = 0;
         double t_single = 0;
@@ -538,8 +548,8 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
             }
         }
     }
-    if (g_ctx.force_config >= 0 && g_ctx.force_config < count) {
-        vi = (int)g_ctx.force_config;
+    if (forced()) {
+        vi = row_by_name(tab, count, g_ctx.force_config);       // (a name this family does not have: unsupported)
         model_split = 0;
     }
     if (vi < 0) return QGEMM_ERR_UNSUPPORTED;
@@ -711,12 +721,7 @@ bool settle_scale_layout(const NtProblem &q, Plan &pl) {
     const Variant *tab = table_for(q.arith, q.block, q.kmaj, &count);
     auto partner = [&](const Variant *v, bool ks) -> const Variant * {      // the row of the pair with / without ASK
         if (v->a_scale_k_contiguous == ks) return v;
-        std::string want = v->name;
-        if (ks) want += "_ks";
-        else if (want.size() > 3) want.resize(want.size() - 3);
-        for (int i = 0; tab && i < count; ++i)
-            if (tab[i].a_scale_k_contiguous == ks && want == tab[i].name) return &tab[i];
-        return nullptr;
+        return (tab && v->twin >= 0 && v->twin < count) ? &tab[v->twin] : nullptr;
     };
     if (q.as_ms == 1) {                                  // rows-contiguous: every kernel but the twins reads that
         for (Plan *p = &pl; p; p = p->rest.get())
@@ -725,17 +730,19 @@ bool settle_scale_layout(const NtProblem &q, Plan &pl) {
     }
     // some other arrangement (K-contiguous, as QGEMM_LAYOUT_K_CONTIGUOUS passes it): fine where every launch of the
     // plan either takes any strides (simple and ping-pong pipelines) or has a twin for it
-    const bool ks_form = q.as_ks == 1 && q.as_ms % 2 == 0 && ((uintptr_t)q.as & 7u) == 0;
+    // (a twin fetches the scales of Variant::ks_blocks K blocks of a row per load, two or four: rows aligned to that
+    // many floats, K and every K slice a multiple of that many blocks)
     bool as_is = true;
-    // (the twin of the row with copying waves takes the scales of four K blocks per copy: rows 16-byte aligned, K and
-    // every K slice a multiple of four blocks)
-    const bool ks4_form = ks_form && q.as_ms % 4 == 0 && ((uintptr_t)q.as & 15u) == 0;
     for (const Plan *p = &pl; as_is && p; p = p->rest.get()) {
         if (p->v->a_scale_any_stride) continue;
         const Variant *twin = partner(p->v, true);
-        as_is = ks_form && twin && !(p->a.nsplit > 1 && p->a.ksteps_per_split % 2 != 0);
-        if (as_is && std::strstr(twin->name, "_cw"))
-            as_is = ks4_form && p->a.ksteps % 4 == 0 && !(p->a.nsplit > 1 && p->a.ksteps_per_split % 4 != 0);
+        if (!twin || q.as_ks != 1) {
+            as_is = false;
+            break;
+        }
+        const uint32_t g = (uint32_t)twin->ks_blocks;
+        as_is = g > 0 && q.as_ms % g == 0 && ((uintptr_t)q.as % (4 * g)) == 0 && p->a.ksteps % g == 0 &&
+                !(p->a.nsplit > 1 && p->a.ksteps_per_split % g != 0);
     }
     for (Plan *p = &pl; p; p = p->rest.get()) {
         if (p->v->a_scale_any_stride) continue;
@@ -929,8 +936,10 @@ QGEMM_EXPORT int qgemm_tile_map(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n,
 QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     if (!key) return QGEMM_ERR_INVALID_ARG;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
-    if (!std::strcmp(key, "force_config")) g_ctx.force_config = value;
-    else if (!std::strcmp(key, "force_split")) g_ctx.force_split = value;
+    if (!std::strcmp(key, "force_config")) {
+        if (value != -1) return QGEMM_ERR_INVALID_ARG;      // rows are named: qgemm_force_config; -1 returns to the heuristic
+        g_ctx.force_config.clear();
+    } else if (!std::strcmp(key, "force_split")) g_ctx.force_split = value;
     else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
     else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
     else if (!std::strcmp(key, "stagger")) g_ctx.stagger = value;
@@ -941,6 +950,44 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
 #endif
     else if (!std::strcmp(key, "row_split")) g_ctx.row_split = value;
     else return QGEMM_ERR_INVALID_ARG;
+    return QGEMM_OK;
+}
+
+QGEMM_EXPORT int qgemm_force_config(const char *name) {
+    std::lock_guard<std::mutex> lock(g_ctx.mu);
+    if (!name || !*name) {
+        g_ctx.force_config.clear();
+        return QGEMM_OK;
+    }
+    // the name has to be a row of at least one family
+    bool known = false;
+    for (int arith = 0; arith < 4 && !known; ++arith)
+        for (int block = 0; block < 2 && !known; ++block)
+            for (int kmaj = 0; kmaj < 4 && !known; ++kmaj) {
+                int count = 0;
+                const Variant *tab = table_for(arith, block != 0, kmaj, &count);
+                known = row_by_name(tab, count, name) >= 0;
+            }
+    if (!known) return QGEMM_ERR_INVALID_ARG;
+    g_ctx.force_config = name;
+    return QGEMM_OK;
+}
+
+QGEMM_EXPORT int qgemm_variant_count(int in_dtype, int scale_mode, int k_major) {
+    int count = 0;
+    const int arith = arith_of(in_dtype);
+    if (arith < 0 || !table_for(arith, scale_mode == QGEMM_SCALE_BLOCK128, k_major, &count)) return 0;
+    return count;
+}
+
+QGEMM_EXPORT int qgemm_variant_name(int in_dtype, int scale_mode, int k_major, int index, char *buf, size_t buflen) {
+    if (!buf || buflen == 0) return QGEMM_ERR_INVALID_ARG;
+    int count = 0;
+    const int arith = arith_of(in_dtype);
+    const Variant *tab = arith < 0 ? nullptr : table_for(arith, scale_mode == QGEMM_SCALE_BLOCK128, k_major, &count);
+    if (!tab) return QGEMM_ERR_UNSUPPORTED;
+    if (index < 0 || index >= count) return QGEMM_ERR_INVALID_ARG;
+    std::snprintf(buf, buflen, "%s", tab[index].name);
     return QGEMM_OK;
 }
 
@@ -1300,14 +1347,18 @@ QGEMM_EXPORT int qgemm_reserve_workspace(size_t bytes) {
     int st = ensure_init_locked();
     if (st != QGEMM_OK) return st;
     if (bytes <= g_ctx.ws.bytes) return QGEMM_OK;
+    // (takes no stream, so it cannot tell whether one is being captured: the caller reserves before a capture)
+    // grow geometrically, as ensure_workspace_locked does: a caller that reserves step by step then retires
+    // O(log n) blocks, not one per call
+    const size_t want = std::max(bytes, 2 * g_ctx.ws.bytes);
     void *p = nullptr;
-    if (hipMalloc(&p, bytes) != hipSuccess) {
+    if (hipMalloc(&p, want) != hipSuccess) {
         (void)hipGetLastError();
         return QGEMM_ERR_ALLOC;
     }
     if (g_ctx.ws.p) g_ctx.retired.push_back(g_ctx.ws.p);
     g_ctx.ws.p = p;
-    g_ctx.ws.bytes = bytes;
+    g_ctx.ws.bytes = want;
     return QGEMM_OK;
 }
 

@@ -47,6 +47,9 @@ SIGNATURES = {
     "qgemm_tile_map": (_i, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32),
                             C.POINTER(C.c_uint32)]),
     "qgemm_set_option": (_i, [C.c_char_p, C.c_long]),
+    "qgemm_force_config": (_i, [C.c_char_p]),
+    "qgemm_variant_count": (_i, [_i, _i, _i]),
+    "qgemm_variant_name": (_i, [_i, _i, _i, _i, C.c_char_p, _sz]),
     "qgemm_last_config": (_i, [C.c_char_p, _sz]),
     "qgemm_plan": (_i, [_i, _i, _i, _sz, _sz, _sz, C.c_char_p, _sz]),
     "qgemm_selftest_layouts": (_i, [C.c_char_p, _sz]),

@@ -49,6 +49,22 @@ def set_option(key, value):
     check(load_library().qgemm_set_option(key.encode(), int(value)))
 
 
+def force_config(name=None):
+    """Pin the row `name` of the variant tables for the GEMM calls that follow (None: back to the heuristic)."""
+    check(load_library().qgemm_force_config(name.encode() if name else None))
+
+
+def variant_names(in_dtype, scale_mode=0, k_major=0):
+    """Names of the rows of the family that serves (in_dtype, scale_mode, k_major); arguments as for plan()."""
+    lib = load_library()
+    out = []
+    for i in range(lib.qgemm_variant_count(in_dtype, scale_mode, k_major)):
+        buf = C.create_string_buffer(64)
+        check(lib.qgemm_variant_name(in_dtype, scale_mode, k_major, i, buf, 64))
+        out.append(buf.value.decode())
+    return out
+
+
 def plan(in_dtype, scale_mode, k_major, M, N, K):
     """Name of the kernel configuration the library would choose (no launch, no device needed)."""
     buf = C.create_string_buffer(128)

@@ -49,14 +49,33 @@ int main(void) {
     CHECK(qgemm_plan(QGEMM_DT_F8E4M3, 1, 0, 0, 1, 1, buf, sizeof buf) == QGEMM_ERR_INVALID_ARG);
     CHECK(qgemm_plan(QGEMM_DT_F8E4M3, 1, 0, 1, 1, 1, NULL, 0) == QGEMM_ERR_INVALID_ARG);
     CHECK(qgemm_plan(99, 1, 0, 1, 1, 1, buf, sizeof buf) == QGEMM_ERR_UNSUPPORTED);
-    /* forced rows and splits through the option table */
-    for (long v = -1; v < 26; ++v) {
-        CHECK(qgemm_set_option("force_config", v) == QGEMM_OK);
-        for (long sp = 0; sp <= 4; ++sp) {
-            CHECK(qgemm_set_option("force_split", sp) == QGEMM_OK);
-            CHECK(qgemm_plan(QGEMM_DT_F8E4M3, QGEMM_SCALE_BLOCK128, 0, 300, 520, 1280, buf, sizeof buf) == QGEMM_OK);
-            CHECK(qgemm_plan(QGEMM_DT_I8, QGEMM_SCALE_PER_MATRIX, 0, 64, 7168, 2048, buf, sizeof buf) == QGEMM_OK);
+    /* forced rows (by name, every row of the two families below) and splits through the option table */
+    {
+        const int nb = qgemm_variant_count(QGEMM_DT_F8E4M3, QGEMM_SCALE_BLOCK128, 0);
+        const int ni = qgemm_variant_count(QGEMM_DT_I8, QGEMM_SCALE_PER_MATRIX, 0);
+        CHECK(nb > 4 && ni > 4 && qgemm_variant_count(99, 1, 0) == 0 && qgemm_variant_count(QGEMM_DT_I8, QGEMM_SCALE_BLOCK128, 0) == 0);
+        CHECK(qgemm_variant_name(QGEMM_DT_I8, 1, 0, ni, buf, sizeof buf) == QGEMM_ERR_INVALID_ARG);
+        CHECK(qgemm_variant_name(QGEMM_DT_I8, 1, 0, 0, NULL, 0) == QGEMM_ERR_INVALID_ARG);
+        for (int v = 0; v < nb + ni; ++v) {
+            char name[64], other[64];
+            const int blockfam = v < nb;
+            CHECK(qgemm_variant_name(blockfam ? QGEMM_DT_F8E4M3 : QGEMM_DT_I8, blockfam ? QGEMM_SCALE_BLOCK128 : QGEMM_SCALE_PER_MATRIX,
+                                     0, blockfam ? v : v - nb, name, sizeof name) == QGEMM_OK && strlen(name) > 0);
+            CHECK(qgemm_force_config(name) == QGEMM_OK);
+            for (long sp = 0; sp <= 4; ++sp) {
+                CHECK(qgemm_set_option("force_split", sp) == QGEMM_OK);
+                /* a family without a row of that name refuses, the one that has it plans it */
+                int st = qgemm_plan(QGEMM_DT_F8E4M3, QGEMM_SCALE_BLOCK128, 0, 300, 520, 1280, buf, sizeof buf);
+                CHECK(st == QGEMM_OK || st == QGEMM_ERR_UNSUPPORTED);
+                if (blockfam) CHECK(st == QGEMM_OK && strlen(buf) >= 3);      /* (the name may be the row's twin for the other a_scale arrangement) */
+                st = qgemm_plan(QGEMM_DT_I8, QGEMM_SCALE_PER_MATRIX, 0, 64, 7168, 2048, other, sizeof other);
+                CHECK(st == QGEMM_OK || st == QGEMM_ERR_UNSUPPORTED);
+                if (!blockfam) CHECK(st == QGEMM_OK && strncmp(other, name, strlen(name)) == 0);
+            }
         }
+        CHECK(qgemm_force_config("no_such_row") == QGEMM_ERR_INVALID_ARG);
+        CHECK(qgemm_set_option("force_config", 3) == QGEMM_ERR_INVALID_ARG);
+        CHECK(qgemm_force_config(NULL) == QGEMM_OK && qgemm_force_config("") == QGEMM_OK);
     }
     CHECK(qgemm_set_option("force_config", -1) == QGEMM_OK && qgemm_set_option("force_split", 0) == QGEMM_OK);
     CHECK(qgemm_set_option("no_such_option", 1) == QGEMM_ERR_INVALID_ARG && qgemm_set_option(NULL, 1) == QGEMM_ERR_INVALID_ARG);

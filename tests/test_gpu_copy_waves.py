@@ -13,7 +13,7 @@ from oracle import cpu_ref as R
 from tests.util import dev, fp8_tensor, host, say, scalar
 
 pytestmark = pytest.mark.gpu
-ROW = 24                                                     # row of the variant table
+ROW = "256x128_w2x2_cw"                                      # row of the variant table
 
 
 @pytest.fixture(autouse=True)
@@ -33,7 +33,7 @@ def test_every_number_of_k_steps(fam):
             for split in ((1, 2) if ksteps >= 4 else (1,)):
                 K = ksteps * (64 if fam.startswith("bf16") else 128)
                 say("copying waves", fam, (M, N, K), "split", split)
-                Q.set_option("force_config", ROW)
+                Q.force_config(ROW)
                 Q.set_option("force_split", split)
                 Q.set_option("kmajor", 2)                    # K-major operands as stored, whatever the estimate says
                 rng = np.random.default_rng(100 * ksteps + split)
@@ -80,7 +80,7 @@ def test_192_row_tile_every_number_of_k_steps(fam):
             for split in ((1, 2) if ksteps >= 4 else (1,)):
                 K = ksteps * (64 if fam == "bf16" else 128)
                 say("192-row tile", fam, (M, N, K), "split", split)
-                Q.set_option("force_config", 26)
+                Q.force_config("192x256_w2x4_solo8")
                 Q.set_option("force_split", split)
                 rng = np.random.default_rng(300 * ksteps + split)
                 a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)

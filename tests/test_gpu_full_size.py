@@ -57,11 +57,11 @@ def test_cfg2_int8_4096_bit_exact():
     assert np.array_equal(got[rows], R.gemm_i8_i32(qa[rows], qb)), name0
     assert np.array_equal(got[:, cols], R.gemm_i8_i32(qa, qb[cols])), name0
     # another tile configuration and a K split: the same integers everywhere
-    Q.set_option("force_config", 2)
+    Q.force_config("128x128_w2x2_dma")
     c2 = torch.zeros_like(c)
     Q.int8_mm(da, db_, scalar(sa), scalar(sb), c2)
     assert Q.last_config() != name0 and torch.equal(c, c2)
-    Q.set_option("force_config", -1)
+    Q.force_config(None)
     c3 = torch.zeros_like(c)
     Q.int8_mm(da, db_, scalar(sa), scalar(sb), c3, split_k=4)
     assert "splitk" in Q.last_config() and torch.equal(c, c3)
@@ -93,7 +93,7 @@ def test_cfg3_fp8_per_matrix_8192():
     c2 = torch.zeros_like(c)
     Q.scaled_gemm(da, db_, scalar(2 * sa), scalar(sb), c2, M, N, K, Q.SCALE_PER_MATRIX)
     assert torch.equal(c2.float(), 2 * c.float())              # power-of-two scale: exact
-    Q.set_option("force_config", 0)
+    Q.force_config("256x256_w2x4_solo8")
     c3 = torch.zeros_like(c)
     Q.scaled_gemm(da, db_, scalar(sa), scalar(sb), c3, M, N, K, Q.SCALE_PER_MATRIX)
     assert Q.last_config() != name0
@@ -310,8 +310,8 @@ def test_one_round_of_256x128_tiles_int8_and_block_scales():
     rows, cols = _sample(M, 32, 3), _sample(N, 32, 4)
     assert np.array_equal(got[rows], R.gemm_i8_i32(qa[rows], qb))
     assert np.array_equal(got[:, cols], R.gemm_i8_i32(qa, qb[cols]))
-    for force, split in ((2, 1), (24, 2)):
-        Q.set_option("force_config", force)
+    for force, split in (("128x128_w2x2_dma", 1), ("256x128_w2x2_cw", 2)):
+        Q.force_config(force)
         Q.set_option("force_split", split)
         c2 = torch.zeros_like(c)
         Q.int8_mm(da, db_, scalar(sa), scalar(sb), c2)

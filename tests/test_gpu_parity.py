@@ -14,16 +14,25 @@ from tests.util import (assert_close, dev, fp8_inputs, fp8_tensor, host, int8_in
 
 pytestmark = pytest.mark.gpu
 
-N_VARIANTS = 28         # rows of the variant table in qgemm_amd/csrc/gemm_inst.hip
+# rows of the variant tables, by name, as the library reports them (one table per family)
+I8_ROWS = Q.variant_names(Q.DT_I8, Q.SCALE_PER_MATRIX)
+F8_ROWS = Q.variant_names(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX)
+F8B_ROWS = Q.variant_names(Q.DT_F8E4M3, Q.SCALE_BLOCK128)
+F8B_TN_ROWS = Q.variant_names(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3)
+ROWS_16 = {"bf16": Q.variant_names(Q.DT_BF16), "f16": Q.variant_names(Q.DT_F16)}
+ROWS_16_NN = {"bf16": Q.variant_names(Q.DT_BF16, 0, 2), "f16": Q.variant_names(Q.DT_F16, 0, 2)}
+PAIRS_16 = [(d, v) for d in ("f16", "bf16") for v in ROWS_16[d]]
+PAIRS_16_NN = [(d, v) for d in ("f16", "bf16") for v in ROWS_16_NN[d]]
 
 
 @pytest.fixture(autouse=True)
 def _reset_options():
     yield
-    Q.set_option("force_config", -1)
+    Q.force_config(None)
     Q.set_option("force_split", 0)
     Q.set_option("group_m", 0)
     Q.set_option("kmajor", 1)
+    Q.set_option("k_rot", -1)
 
 
 def test_selftest_layouts():
@@ -38,14 +47,14 @@ def test_selftest_layouts():
 
 
 # ----------------------------------------------------------------- int8
-@pytest.mark.parametrize("variant", range(N_VARIANTS))
+@pytest.mark.parametrize("variant", I8_ROWS)
 @pytest.mark.parametrize("shape", [(256, 256, 256), (300, 202, 384), (16, 128, 128), (520, 1000, 640)])
 def test_int8_accumulators_bit_exact_every_variant(variant, shape):
     M, N, K = shape
     say("int8 i32", shape, "variant", variant)
-    qa, sa, qb, sb = int8_inputs(M, N, K, seed=100 + variant)
+    qa, sa, qb, sb = int8_inputs(M, N, K, seed=100 + I8_ROWS.index(variant))
     ref = R.gemm_i8_i32(qa, qb)
-    Q.set_option("force_config", variant)
+    Q.force_config(variant)
     c = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
     Q.int8_mm(dev(qa), dev(qb), scalar(sa), scalar(sb), c, split_k=1)
     assert np.array_equal(host(c), ref), Q.last_config()
@@ -88,13 +97,13 @@ def test_int8_split_k_bit_exact(nsplit):
 
 
 # ------------------------------------------------------------------ fp8
-@pytest.mark.parametrize("variant", range(N_VARIANTS))
+@pytest.mark.parametrize("variant", F8_ROWS)
 def test_fp8_per_matrix_every_variant(variant):
     M, N, K = 272, 392, 512
     say("fp8 per-matrix", (M, N, K), "variant", variant)
-    qa, sa, qb, sb = fp8_inputs(M, N, K, seed=200 + variant)
+    qa, sa, qb, sb = fp8_inputs(M, N, K, seed=200 + F8_ROWS.index(variant))
     ref = R.gemm_f32acc(R.decode_fp8(qa), R.decode_fp8(qb)) * np.float32(sa * sb)
-    Q.set_option("force_config", variant)
+    Q.force_config(variant)
     for dt in (torch.bfloat16, torch.float32, torch.float16):
         c = torch.zeros((M, N), dtype=dt, device="cuda")
         Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), scalar(sa), scalar(sb), c, M, N, K, Q.SCALE_PER_MATRIX,
@@ -133,24 +142,24 @@ def test_fp8_every_code_decodes_like_the_oracle():
     assert np.array_equal(np.diag(got)[: len(codes)], R.decode_fp8(codes))
 
 
-@pytest.mark.parametrize("variant", range(N_VARIANTS))
+@pytest.mark.parametrize("variant", F8B_ROWS)
 def test_fp8_block_scaled_every_variant(variant):
     M, N, K = 160, 384, 512
     say("fp8 block-scaled", (M, N, K), "variant", variant)
-    qa, _, qb, _ = fp8_inputs(M, N, K, seed=300 + variant)
+    qa, _, qb, _ = fp8_inputs(M, N, K, seed=300 + F8B_ROWS.index(variant))
     as_ = R.fill_uniform((M, K // 128), 301, 0.5, 2.0)
     bs = R.fill_uniform((N // 128, K // 128), 302, 0.5, 2.0)
     # bring the products to O(1) so atol means something
     as_ *= np.float32(1.0 / 448.0)
     bs *= np.float32(1.0 / 448.0)
     ref = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)
-    Q.set_option("force_config", variant)
+    Q.force_config(variant)
     c = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
     Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128, split_k=1)
     assert_close(host(c), ref, what=Q.last_config())
 
 
-@pytest.mark.parametrize("variant", [-1] + list(range(N_VARIANTS)))
+@pytest.mark.parametrize("variant", [None] + F8B_ROWS)
 @pytest.mark.parametrize("shape", [(64, 256, 512), (272, 392, 768)])
 def test_fp8_block_scaled_power_of_two_scales_bit_exact(variant, shape):
     """Power-of-two scales commute exactly with fp32 arithmetic, and small-integer products sum exactly:
@@ -158,8 +167,8 @@ def test_fp8_block_scaled_power_of_two_scales_bit_exact(variant, shape):
     index, row or K block, cannot hide behind a tolerance).  Ragged M and N in the second shape."""
     M, N, K = shape
     say("fp8 block pow2", shape, "variant", variant)
-    Q.set_option("force_config", variant)
-    rng = np.random.default_rng(6 + variant)
+    Q.force_config(variant)
+    rng = np.random.default_rng(6 + ([None] + F8B_ROWS).index(variant))
     a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
     b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
     as_ = (2.0 ** rng.integers(-3, 4, size=(M, K // 128))).astype(np.float32)
@@ -167,7 +176,7 @@ def test_fp8_block_scaled_power_of_two_scales_bit_exact(variant, shape):
     ref = R.gemm_fp8_block(a, b, as_, bs)
     c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K,
-                  Q.SCALE_BLOCK128, split_k=1 if variant >= 0 else 0)
+                  Q.SCALE_BLOCK128, split_k=1 if variant else 0)
     assert np.array_equal(host(c), ref), Q.last_config()
 
 
@@ -186,7 +195,7 @@ def test_fp8_block_scaled_k_contiguous_scale_twin(case):
     as_ = (2.0 ** rng.integers(-3, 4, size=(M, K // 128))).astype(np.float32)
     bs = (2.0 ** rng.integers(-3, 4, size=((N + 127) // 128, K // 128))).astype(np.float32)
     ref = R.gemm_fp8_block(a, b, as_, bs)
-    Q.set_option("force_config", 12)
+    Q.force_config("256x256_w2x4_solo8")
     Q.set_option("force_split", split)
     c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
@@ -224,7 +233,7 @@ def test_fp8_mm_reference_layout():
     assert np.array_equal(tn, ref)
 
 
-@pytest.mark.parametrize("variant", range(N_VARIANTS))
+@pytest.mark.parametrize("variant", F8B_TN_ROWS)
 @pytest.mark.parametrize("shape", [(160, 224, 512), (288, 544, 384)])
 def test_fp8_mm_reference_layout_native_every_variant(variant, shape):
     """The reference storage (A is K x M, B is K x N, hip_mix_gemm_kernel.cpp:96,111) read as it lies, through
@@ -232,7 +241,7 @@ def test_fp8_mm_reference_layout_native_every_variant(variant, shape):
     the route through the transpose utility (same kernel arithmetic, other summation order inside an MFMA)."""
     M, N, K = shape
     say("fp8_mm reference layout, native", shape, "variant", variant)
-    qa, _, qb, _ = fp8_inputs(M, N, K, seed=500 + variant)
+    qa, _, qb, _ = fp8_inputs(M, N, K, seed=500 + F8B_TN_ROWS.index(variant))
     as_ = R.fill_uniform((M, K // 128), 501, 0.5, 2.0) / np.float32(448)
     bs = R.fill_uniform(((N + 127) // 128, K // 128), 502, 0.5, 2.0) / np.float32(448)
     ref = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)
@@ -240,10 +249,10 @@ def test_fp8_mm_reference_layout_native_every_variant(variant, shape):
     b_t = fp8_tensor(np.ascontiguousarray(qb.T)).t()
     as_t = dev(np.ascontiguousarray(as_.T)).t()
     bs_t = dev(np.ascontiguousarray(bs.T)).t()
-    Q.set_option("force_config", variant)
+    Q.force_config(variant)
     c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.fp8_mm(a_t, b_t, as_t, bs_t, c)
-    assert Q.last_config().endswith("_tn"), Q.last_config()
+    assert Q.last_config() == variant + "_tn", Q.last_config()
     assert_close(host(c), ref, what=Q.last_config())
     Q.set_option("kmajor", 0)
     c2 = torch.zeros_like(c)
@@ -329,6 +338,91 @@ def test_fp8_split_k(nsplit):
     assert_close(host(c), refb)
 
 
+def _stratified_f32():
+    """fp32 bit patterns that exercise a narrowing conversion: NaNs, infinities, zeros, fp32 subnormals, exact ties
+    of the bf16 rounding (low half 0x8000 under an even and an odd upper half) and their neighbours, the fp16
+    overflow boundary (65504, 65520 and neighbours), the fp16 subnormal range with its ties, and random patterns
+    of every exponent."""
+    rng = np.random.default_rng(2024)
+    bits = [0x7FC00000, 0xFFC00000, 0x7F800001, 0x7FFFFFFF, 0x7F800000, 0xFF800000, 0x00000000, 0x80000000,
+            0x00000001, 0x80000001, 0x007FFFFF, 0x00008000, 0x00018000, 0x7F7FFFFF, 0xFF7FFFFF, 0x7F7F8000, 0x7F7F7FFF]
+    for upper in (0x3F80, 0x3F81, 0x4049, 0xC2F7, 0x0001, 0x0002, 0x7F7E):
+        for low in (0x7FFF, 0x8000, 0x8001, 0x0000, 0xFFFF):
+            bits.append((upper << 16) | low)
+    for v in (65504.0, 65519.996, 65520.0, 65536.0, 1e9, -65519.996, -65520.0):
+        bits.append(int(np.float32(v).view(np.uint32)))
+    for e in range(-26, -13):                       # fp16 subnormals and the smallest normals: quarter steps and ties
+        for m in (1.0, 1.25, 1.5, 1.75, 1.0009765625, 1.00048828125, 1.001464843750):
+            for sgn in (1.0, -1.0):
+                bits.append(int(np.float32(sgn * m * 2.0 ** e).view(np.uint32)))
+    rnd = rng.integers(0, 1 << 32, size=3600, dtype=np.uint64).astype(np.uint32)
+    all_bits = np.concatenate([np.array(bits, np.uint64).astype(np.uint32), rnd])
+    return all_bits.view(np.float32)
+
+
+@pytest.mark.parametrize("variant", [None, "256x256_w2x4_solo8", "128x128_w2x2_dma", "skinny_128x32_k8", "256x128_w2x2_cw"])
+def test_epilogue_conversions_match_the_oracle_codecs(variant):
+    """The float -> bf16 / fp16 conversion of the epilogues (f32_to_bf16_bits / f32_to_f16_bits, csrc/common.h: the
+    NaN-guarded form of src/include/fast_quat.h:3-12) on a stratified fp32 sample, bit for bit against the oracle's
+    codecs.  The sample travels as a_scale of a block-scaled GEMM whose only product per row is 1.0 * 1.0, so that
+    the accumulator the epilogue converts is exactly the sample value (fma(1, x, 0) = x)."""
+    x = _stratified_f32()
+    M, N, K = len(x), 128, 128
+    say("epilogue conversions", (M, N, K), "variant", variant)
+    qa = np.zeros((M, K), np.uint8)
+    qa[:, 0] = 0x38                                  # 1.0
+    qb = np.zeros((N, K), np.uint8)
+    qb[:, 0] = 0x38
+    as_ = x.reshape(M, 1).copy()
+    bs = np.ones((1, 1), np.float32)
+    with np.errstate(all="ignore"):
+        acc = x + np.float32(0.0)                    # what the fold leaves: -0 becomes +0, everything else is itself
+    nan = np.isnan(acc)
+    Q.force_config(variant)
+    for dt, enc in ((torch.bfloat16, R.encode_bf16), (torch.float16, R.encode_f16), (torch.float32, None)):
+        c = torch.zeros((M, N), dtype=dt, device="cuda")
+        Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128, split_k=1)
+        torch.cuda.synchronize()
+        if enc is None:
+            got = c.cpu().numpy()
+            assert np.array_equal(got[~nan].view(np.uint32), np.broadcast_to(acc[:, None], got.shape)[~nan].view(np.uint32))
+            assert np.all(np.isnan(got[nan]))
+            continue
+        got = c.view(torch.int16).cpu().numpy().view(np.uint16)
+        want = enc(acc)
+        bad = (got[~nan] != want[~nan, None])
+        assert not bad.any(), (Q.last_config(), dt, [hex(int(v)) for v in acc[~nan].view(np.uint32)[np.nonzero(bad.any(axis=1))[0][:8]]])
+        # NaN in, NaN out (payload free): exponent all ones, mantissa non-zero
+        g = got[nan].astype(np.uint32)
+        if dt == torch.bfloat16:
+            assert np.all(((g & 0x7F80) == 0x7F80) & ((g & 0x007F) != 0))
+        else:
+            assert np.all(((g & 0x7C00) == 0x7C00) & ((g & 0x03FF) != 0))
+
+
+def test_rotated_k_start_changes_only_the_summation_order():
+    """With at most 256 rows the workgroups of column tile i start their K loops 3 i steps in (option "k_rot"): the
+    same products summed in another order.  Random fp8 data: with and without the rotation the results agree to the
+    stated tolerance with the oracle and to a few fp32 ulps of the sum's magnitude with each other; identical rows of
+    A against identical columns of B give identical bits at every column position only with k_rot = 0."""
+    M, N, K = 64, 1024, 4096
+    say("k_rot on / off", (M, N, K))
+    qa, sa, qb1, sb = fp8_inputs(M, 128, K, seed=77)
+    qb = np.tile(qb1, (N // 128, 1))                 # every 128-column block of B holds the same columns
+    ref = R.gemm_f32acc(R.decode_fp8(qa), R.decode_fp8(qb)) * np.float32(sa * sb)
+    out = {}
+    for rot in (-1, 0):
+        Q.set_option("k_rot", rot)
+        c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), scalar(sa), scalar(sb), c, M, N, K, Q.SCALE_PER_MATRIX)
+        out[rot] = host(c)
+        assert_close(out[rot], ref, what=f"k_rot {rot} {Q.last_config()}")
+    Q.set_option("k_rot", -1)
+    assert np.max(np.abs(out[-1] - out[0])) <= 1e-4 * np.max(np.abs(ref))
+    blocks0 = out[0].reshape(M, N // 128, 128)
+    assert np.array_equal(blocks0, np.broadcast_to(blocks0[:, :1], blocks0.shape))     # position-independent sums
+
+
 # ---------------------------------------------------------- plain fp16 / bf16
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("layout_b", ["nk", "kn"])
@@ -352,8 +446,7 @@ def test_plain_gemm_16bit(dtype, layout_b, shape):
         assert_close(got, ref, rtol=rtol, atol=1e-3, what=f"{Q.last_config()} {out_dt}")
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("variant", range(N_VARIANTS))
+@pytest.mark.parametrize("dtype,variant", PAIRS_16)
 def test_plain_gemm_16bit_every_variant(dtype, variant):
     """Every tile variant on 16-bit operands (the big tiles use the 32 x 32 x 16 MFMA and their own fragment and
     accumulator layouts): small integers, so sums are exact and the bits must equal numpy's integer product,
@@ -361,11 +454,11 @@ def test_plain_gemm_16bit_every_variant(dtype, variant):
     M, N, K = 300, 328, 384
     say("plain 16-bit", dtype, "variant", variant)
     tdt = torch.float16 if dtype == "f16" else torch.bfloat16
-    rng = np.random.default_rng(40 + variant)
+    rng = np.random.default_rng(40 + ROWS_16[dtype].index(variant))
     a = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
     b = rng.integers(-4, 5, size=(N, K)).astype(np.float32)
     ref = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)       # |ref| <= 16 * 384: exact in fp32
-    Q.set_option("force_config", variant)
+    Q.force_config(variant)
     c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.gemm(torch.from_numpy(a).cuda().to(tdt), torch.from_numpy(b).cuda().to(tdt), c, "nk")
     assert np.array_equal(host(c), ref), Q.last_config()
@@ -380,8 +473,7 @@ def test_plain_gemm_16bit_every_variant(dtype, variant):
     assert torch.equal(c2.cpu(), ref2), Q.last_config()
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("variant", range(N_VARIANTS))
+@pytest.mark.parametrize("dtype,variant", PAIRS_16_NN)
 def test_plain_gemm_nn_native_every_variant(dtype, variant):
     """GEMM_kernel_v1..v5 storage (B is K x N, include/gemm.h:25-66) read as it lies through the K-major B tile,
     every tile variant, ragged M and N, a padded leading dimension of B, against the oracle."""
@@ -389,15 +481,15 @@ def test_plain_gemm_nn_native_every_variant(dtype, variant):
     say("plain NN native", dtype, "variant", variant)
     enc, dec, tdt = ((R.encode_f16, R.decode_f16, torch.float16) if dtype == "f16"
                      else (R.encode_bf16, R.decode_bf16, torch.bfloat16))
-    ha, hb = enc(R.fill_uniform((M, K), 71 + variant)), enc(R.fill_uniform((K, N), 72))
+    ha, hb = enc(R.fill_uniform((M, K), 71 + ROWS_16_NN[dtype].index(variant))), enc(R.fill_uniform((K, N), 72))
     ref = R.gemm_f32acc(dec(ha), dec(hb), "nn")
     a = dev(ha.view(np.int16)).view(tdt)
     b_pad = torch.full((K, ldB), 7.0, dtype=tdt, device="cuda")          # columns N .. ldB-1 must never matter
     b_pad[:, :N] = dev(hb.view(np.int16)).view(tdt)
-    Q.set_option("force_config", variant)
+    Q.force_config(variant)
     c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.gemm(a, b_pad[:, :N], c, "kn")
-    assert Q.last_config().endswith("_nn"), Q.last_config()
+    assert Q.last_config() == variant + "_nn", Q.last_config()
     assert_close(host(c), ref, rtol=1e-5, atol=1e-3, what=Q.last_config())
     # the route through the transpose utility needs ldB == N
     Q.set_option("kmajor", 0)
