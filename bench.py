@@ -206,7 +206,8 @@ def one_shape(Q, torch, dev, spec, launches):
         fn = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)
     elif fam == "fp8block":
         a, _ = _quant_fp8(torch.randn(M, K, device=dev)); b, _ = _quant_fp8(torch.randn(N, K, device=dev))
-        sa = (torch.rand(M, K // 128, device=dev) + 0.5) / 448; sb = (torch.rand((N + 127) // 128, K // 128, device=dev) + 0.5) / 448
+        KB = (K + 127) // 128
+        sa = (torch.rand(M, KB, device=dev) + 0.5) / 448; sb = (torch.rand((N + 127) // 128, KB, device=dev) + 0.5) / 448
         fn = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_BLOCK128)
     elif fam == "int8":
         a, sa = _quant_i8(torch.randn(M, K, device=dev)); b, sb = _quant_i8(torch.randn(N, K, device=dev))
@@ -510,7 +511,18 @@ def main():
         c4 = torch.empty(m4, n4, dtype=torch.bfloat16, device=dev)
         extra["cfg4_fp8_block_6144x4608x7168"] = gemm_entry(
             tx(lambda: Q.scaled_gemm(a4, b4, as4, bs4, c4, m4, n4, k4, Q.SCALE_BLOCK128)), f4, PEAK_TFLOPS["f8"])
-        del a4, b4, c4
+        del a4, b4
+        # the same shape with K = 7200: 56 whole K blocks and a quarter of one (K % 32 == 0 is all the reference's
+        # dispatch asks for); rows of 7200 bytes are not 128-byte aligned, so every K step of a row spans two lines
+        k4t = 7200
+        a4t, _ = _quant_fp8(torch.randn(m4, k4t, device=dev))
+        b4t, _ = _quant_fp8(torch.randn(n4, k4t, device=dev))
+        kb4t = (k4t + 127) // 128
+        as4t = torch.rand(m4, kb4t, device=dev) * 1.5 + 0.5
+        bs4t = torch.rand(n4 // 128, kb4t, device=dev) * 1.5 + 0.5
+        extra["cfg4_shape_k7200_partial_last_k_block"] = gemm_entry(
+            tx(lambda: Q.scaled_gemm(a4t, b4t, as4t, bs4t, c4, m4, n4, k4t, Q.SCALE_BLOCK128)), 2.0 * m4 * n4 * k4t, PEAK_TFLOPS["f8"])
+        del a4t, b4t, c4
         # cfg 5: skinny M, N = 7168, K = 2048, int8 (f32 out) and fp8 (bf16 out); bandwidth-bound: GB/s of algorithmic
         # bytes.  "rotated": every launch of the graph reads another B (24 buffers, 352 MB: more than the Infinity
         # Cache holds); "resident": all 24 launches read the same B.

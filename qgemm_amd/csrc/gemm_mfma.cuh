@@ -55,7 +55,8 @@ struct GemmArgs {
     const float *as;      // per-matrix: 1 float; block: as[m*as_ms + kb*as_ks]
     const float *bs;      // per-matrix: 1 float; block: bs[nb*bs_ns + kb*bs_ks]
     uint32_t M, N;
-    uint32_t ksteps;      // K steps of 128 bytes in total
+    uint32_t ksteps;      // K steps of 128 bytes in total, the last one possibly partial
+    uint32_t k_tail;      // bytes of K in the last step when it is partial (a multiple of 16), 0 when it is whole
     uint32_t lda, ldb;    // bytes
     uint32_t ldc;         // elements
     uint32_t tiles_m, tiles_n, group_m;
@@ -328,11 +329,17 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     // that are not stored.
     const uint32_t a_rows = p.M - row0 < (uint32_t)C::BM ? p.M - row0 : C::BM;
     const uint32_t b_rows = p.N - col0 < (uint32_t)C::BN ? p.N - col0 : C::BN;
-    const uint32_t kbytes = (uint32_t)nk * C::BKB;
+    // A partial last K step (K bytes not a multiple of 128; the slice that ends with the last step has it): the
+    // ranges end with the last byte of K, and in that one step the lanes whose 16-byte chunk of a K-contiguous row
+    // lies past the end of the row present an offset that is out of range (bit 31; the host keeps every valid
+    // offset below 2^31 for such shapes), so the DMA writes zeros where the next row's bytes would have landed.
+    // A K-major operand needs nothing: its k rows past the end of K lie past the end of the range.
+    const bool has_tail = p.k_tail != 0 && kend == p.ksteps && nk > 0;
+    const uint32_t kbytes = has_tail ? (uint32_t)(nk - 1) * C::BKB + p.k_tail : (uint32_t)nk * C::BKB;
     // K-major operand: rows are k (stride lda / ldb bytes), the tile starts at column row0 / col0; the range ends
     // with the last column of the last k row of this K slice.  Columns past M / N inside an earlier row read
     // the neighbouring row instead (valid memory) and, as above, only feed outputs that are not stored.
-    const uint32_t krows = nk > 0 ? (uint32_t)nk * C::KE : 1;
+    const uint32_t krows = nk > 0 ? kbytes / C::ES : 1;
     const __amdgpu_buffer_rsrc_t ra =
         C::KMA ? make_rsrc(p.A + (size_t)kbeg * C::KE * p.lda + (size_t)row0 * C::ES,
                            (krows - 1) * p.lda + (p.M - row0) * C::ES)
@@ -359,6 +366,10 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     const int ld_chunk_km = (lane & 7) ^ kmajor_swz<C::ES>(ld_r + 16 * ((lw >> 1) & 1));
     const uint32_t voff_a = ld_r * p.lda + (C::KMA ? ld_chunk_km : ld_chunk) * 16;
     const uint32_t voff_b = ld_r * p.ldb + (C::KMB ? ld_chunk_km : ld_chunk) * 16;
+    // (the chunk of a lane is the same in every copy instruction of every pipeline: (lane & 7) - (lane >> 3) mod 8)
+    const uint32_t tail_or = (has_tail && (uint32_t)ld_chunk * 16 >= p.k_tail) ? 0x80000000u : 0u;
+    const uint32_t voff_a_t = C::KMA ? voff_a : (voff_a | tail_or), voff_b_t = C::KMB ? voff_b : (voff_b | tail_or);
+    const int kt_tail = has_tail ? nk - 1 : -1;              // the step (of this slice) that is partial
     // K step the loop's step kt stands for (rotated start, simple pipeline only: the pipelined kernels run
     // compute-bound shapes, whose workgroups share panels and should stay in step)
     constexpr bool K_ROT = C::PIPE == PIPE_SIMPLE;
@@ -385,13 +396,15 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 
     auto issue_stage = [&](int kt) {       // global -> LDS
         char *stage = smem + (kt % C::NSTAGE) * C::STAGE_BYTES;
+        const bool tl = kpos(kt) == kt_tail;
+        const uint32_t va = tl ? voff_a_t : voff_a, vb = tl ? voff_b_t : voff_b;
 #pragma unroll
         for (int i = 0; i < C::LPT; ++i) {
             lds_void *dst = (lds_void *)(stage + (wave + i * C::NW) * 1024);
             if (i < LPT_A0)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, load_soff(i, kt), 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, va, load_soff(i, kt), 0, 0);
             else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, load_soff(i, kt), 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, load_soff(i, kt), 0, 0);
         }
     };
 
@@ -537,23 +550,25 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void *)dst, 16, vo, so, 3072, 0); break;
             }
         };
-        auto issue_a1 = [&](int i, int kt, int buf) {
+        // (tor: tail_or when the copy belongs to the partial last K step, else 0: the literal 0 in the unrolled groups
+        // of the K loop, where the OR then costs nothing)
+        auto issue_a1 = [&](int i, int kt, int buf, uint32_t tor) {
             if constexpr (VOFF_PER_COPY) {
                 char *grp = smem + buf * C::A_BYTES + (lw * LPT_A + (i & ~3)) * 1024;
-                dma(ra_g, grp, vo_copy[i], (uint32_t)kt * C::BKB, i & 3);
+                dma(ra_g, grp, vo_copy[i] | tor, (uint32_t)kt * C::BKB, i & 3);
             } else {
                 lds_void *dst = (lds_void *)(smem + buf * C::A_BYTES + (lw + i * C::NW) * 1024);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, load_soff(i, kt), 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, C::KMA ? voff_a : (voff_a | tor), load_soff(i, kt), 0, 0);
             }
         };
-        auto issue_b1 = [&](int i, int kt) {
+        auto issue_b1 = [&](int i, int kt, uint32_t tor) {
             if constexpr (VOFF_PER_COPY) {
                 const int il = i - LPT_A;
                 char *grp = smem + B_BASE + (kt & 1) * C::B_BYTES + (lw * LPT_B + (il & ~3)) * 1024;
-                dma(rb_g, grp, vo_copy[i], (uint32_t)kt * C::BKB, il & 3);
+                dma(rb_g, grp, vo_copy[i] | tor, (uint32_t)kt * C::BKB, il & 3);
             } else {
                 lds_void *dst = (lds_void *)(smem + B_BASE + (kt & 1) * C::B_BYTES + (lw + i * C::NW) * 1024 - C::A_BYTES);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, load_soff(i, kt), 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, C::KMB ? voff_b : (voff_b | tor), load_soff(i, kt), 0, 0);
             }
         };
         auto next_buf = [&](int bufi) { return bufi + 1 == NA_BUF ? 0 : bufi + 1; };
@@ -689,7 +704,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // every other step: the buffer range check turns what lies beyond the operand into zeros, the
             // rest is data nobody reads, and one straight-line loop body serves all steps (a second, guarded
             // copy of the body cost register spills of its own).
-            auto step = [&](int kt, int par) {             // par = kt & 1
+            // (generic_tag: the form of the step outside the unrolled groups.  Only there can the copies a step issues,
+            // those of step kt + 2, be the ones of a partial last K step: they carry the OR that puts the lanes past
+            // the end of K out of range, 0 for every other step.)
+            auto step = [&](int kt, int par, auto generic_tag) {             // par = kt & 1
+                constexpr bool GENERIC = decltype(generic_tag)::value;
+                const uint32_t tor = GENERIC ? (kt + 2 == kt_tail ? tail_or : 0u) : 0u;
                 const int a_nx = next_buf(a_rd);
                 constexpr bool copies = !C::COPYW;            // (the copying waves' loop is below)
                 // block scales of this step (fetched one step ahead) and the fetch for the next one, in front of
@@ -733,12 +753,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     if (a < COPY_ROWS_A) {
 #pragma unroll
                         for (int j = (slot - 2) * CPS_A; j < (slot - 1) * CPS_A; ++j)
-                            if (j < CPR_A && a * CPR_A + j < LPT_A) issue_a1(a * CPR_A + j, kt + 2, a_wr);
+                            if (j < CPR_A && a * CPR_A + j < LPT_A) issue_a1(a * CPR_A + j, kt + 2, a_wr, tor);
                     } else if (a >= BR) {
                         const int r = a - BR;
 #pragma unroll
                         for (int j = (slot - 2) * CPS_B; j < (slot - 1) * CPS_B; ++j)
-                            if (j < CPR_B && r * CPR_B + j < LPT_B) issue_b1(LPT_A + r * CPR_B + j, kt + 2);
+                            if (j < CPR_B && r * CPR_B + j < LPT_B) issue_b1(LPT_A + r * CPR_B + j, kt + 2, tor);
                     }
                 };
                 auto step_barrier = [&]() {
@@ -819,15 +839,16 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 a_wr = next_buf(a_wr);
             };
             auto first_copies = [&]() {
+                const uint32_t tor0 = kt_tail == 0 ? tail_or : 0u, tor1 = kt_tail == 1 ? tail_or : 0u;
 #pragma unroll
-                for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0);
+                for (int i = 0; i < LPT_A; ++i) issue_a1(i, 0, 0, tor0);
 #pragma unroll
-                for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 0);
+                for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 0, tor0);
                 if (nk > 1) {
 #pragma unroll
-                    for (int i = 0; i < LPT_A; ++i) issue_a1(i, 1, 1);
+                    for (int i = 0; i < LPT_A; ++i) issue_a1(i, 1, 1, tor1);
 #pragma unroll
-                    for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 1);
+                    for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, 1, tor1);
                 }
             };
             if constexpr (C::COPYW) {
@@ -856,10 +877,11 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         phase_barrier();
                         int aw = 2;
                         for (int kt = 0; kt < nk; ++kt) {
+                            const uint32_t tor = kt + 2 == kt_tail ? tail_or : 0u;
                             if (kt + 2 < nk) {
                                 if (((kt + 2) & 3) == 0) issue_scale_group(kt + 2);     // older than the A copies: waited for below
 #pragma unroll
-                                for (int i = 0; i < LPT_A; ++i) issue_a1(i, kt + 2, aw);
+                                for (int i = 0; i < LPT_A; ++i) issue_a1(i, kt + 2, aw, tor);
                                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPT_A));
                             } else {
                                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
@@ -867,7 +889,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                             phase_barrier();
                             if (kt + 2 < nk) {
 #pragma unroll
-                                for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, kt + 2);
+                                for (int i = LPT_A; i < C::LPT; ++i) issue_b1(i, kt + 2, tor);
                             }
                             aw = next_buf(aw);
                         }
@@ -894,28 +916,33 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // B(0) is in registers everywhere before step 0 starts to overwrite its buffer
                 __builtin_amdgcn_s_waitcnt(waitcnt_lgkm0());
                 phase_barrier();
+                typedef std::integral_constant<bool, true> yes_t;
+                typedef std::integral_constant<bool, false> no_t;
+                // the step whose copies (for step kt + 2) are those of a partial last step runs in the generic form
+                // below, the only place where the copies carry the OR for the lanes past the end of K
+                const int kt_tailc = kt_tail >= 2 ? kt_tail - 2 : 0x7fffffff;
                 int kt = 0;
                 {
                     // Six steps at a time (the A ring has three buffers, B two): inside the group the buffer of every
                     // read and copy is a constant, so the ring arithmetic (two dozen scalar and vector adds per
                     // step) folds into immediate offsets.  With one wave per SIMD what is not issued is MFMA time
                     // (bf16 -1.2 %, fp8 -1.2 %, int8 -0.8 % on 8192^3); the 8-wave block-scaled kernel gains 1.6 %.
-                    for (; kt + 6 <= nk; kt += 6) {
+                    for (; kt + 6 <= nk && kt + 6 <= kt_tailc; kt += 6) {
 #pragma unroll
                         for (int j = 0; j < 6; ++j) {
                             a_rd = j % 3;
                             a_wr = (j + 2) % 3;
-                            step(kt + j, j & 1);
+                            step(kt + j, j & 1, no_t{});
                         }
                     }
                     a_rd = 0;            // kt is a multiple of six here
                     a_wr = 2;
                 }
                 for (; kt + 2 <= nk; kt += 2) {
-                    step(kt, 0);
-                    step(kt + 1, 1);
+                    step(kt, 0, yes_t{});
+                    step(kt + 1, 1, yes_t{});
                 }
-                if (kt < nk) step(kt, 0);
+                if (kt < nk) step(kt, 0, yes_t{});
                 __builtin_amdgcn_s_waitcnt(0x0070);      // copies landed, reads done, before LDS serves the epilogue
                 phase_barrier();
                 // the MFMAs above are opaque to the compiler's hazard handling: give the last one its wait states
@@ -988,14 +1015,16 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 };
                 auto issue_stage_k2 = [&](int kt) {
                     char *stage = smem + (kt % NS) * C::STAGE_BYTES + pw * 1024;
+                    const bool tl = kpos(kt) == kt_tail;
+                    const uint32_t va = tl ? voff_a_t : voff_a, vb = tl ? voff_b_t : voff_b;
 #pragma unroll
                     for (int j = 0; j < NPC; ++j) {
                         lds_void *dst = (lds_void *)(stage + j * 4096);
                         const uint32_t blk = (pw >> 1) + 2 * j;
                         if (2 * j < C::RBA)
-                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff_a, soff_k2(C::KMA, blk, p.lda, kt), 0, 0);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, va, soff_k2(C::KMA, blk, p.lda, kt), 0, 0);
                         else
-                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, voff_b, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 0);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 0);
                     }
                     if constexpr (C::BLOCK_SCALE) {
                         if (!p.as_groups) {

@@ -94,13 +94,18 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     // steps past the end of K read as zeros.
     const uint32_t a_rows = p.M - row0 < (uint32_t)C::BM ? p.M - row0 : C::BM;
     const uint32_t b_rows = p.N - col0 < (uint32_t)C::BN ? p.N - col0 : C::BN;
-    const uint32_t kbytes = (uint32_t)nk * 128;
+    // (a partial last K step: the ranges end with the last byte of K, and in that step the lanes whose 16-byte chunk
+    // lies past the end of a row present an offset that is out of range, as in gemm_nt_kernel)
+    const bool has_tail = p.k_tail != 0 && kend == p.ksteps && nk > 0;
+    const uint32_t kbytes = has_tail ? (uint32_t)(nk - 1) * 128 + p.k_tail : (uint32_t)nk * 128;
+    const int kt_tail = has_tail ? nk - 1 : -1;
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A + (size_t)row0 * p.lda + (size_t)kbeg * 128, (a_rows - 1) * p.lda + kbytes);
     const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B + (size_t)col0 * p.ldb + (size_t)kbeg * 128, (b_rows - 1) * p.ldb + kbytes);
     // a copy moves 8 rows x 128 bytes; lane l fetches the chunk of row l >> 3 that belongs in 16-byte slot l of
     // the kilobyte (rotation by the row: see lds_slot)
     const uint32_t rot = (((lane & 7) - (lane >> 3)) & 7) * 16;
     const uint32_t voff_a = (lane >> 3) * p.lda + rot, voff_b = (lane >> 3) * p.ldb + rot;
+    const uint32_t tail_or = (has_tail && rot >= p.k_tail) ? 0x80000000u : 0u;
     char *ring = smem + wave * C::RING_BYTES;
     const int fr = lane & 15, fg = lane >> 4;
     const int off0 = lds_slot(fr, fg) * 16, off1 = lds_slot(fr, 4 + fg) * 16;
@@ -116,16 +121,18 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     // copies: n kilobytes of step kt (rows 8 * first ..) of A or B into ring slots slot, slot + 1, ...
     auto copy_a = [&](int kt_loop, int first, int n, int slot) {
         const int kt = kpos(kt_loop);
+        const uint32_t va = kt == kt_tail ? (voff_a | tail_or) : voff_a;
 #pragma unroll
         for (int i = 0; i < n; ++i)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void *)(ring + (slot + i) * 1024), 16, voff_a,
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void *)(ring + (slot + i) * 1024), 16, va,
                                                      (first + i) * 8 * p.lda + (uint32_t)kt * 128, 0, 0);
     };
     auto copy_b_part = [&](int kt_loop, int first, int n, int slot) {
         const int kt = kpos(kt_loop);
+        const uint32_t vb = kt == kt_tail ? (voff_b | tail_or) : voff_b;
 #pragma unroll
         for (int i = 0; i < n; ++i)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void *)(ring + (slot + i) * 1024), 16, voff_b,
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void *)(ring + (slot + i) * 1024), 16, vb,
                                                      (first + i) * 8 * p.ldb + (uint32_t)kt * 128, 0, 0);
     };
     auto copy_b = [&](int kt, int slot) { copy_b_part(kt, 0, C::SB, slot); };

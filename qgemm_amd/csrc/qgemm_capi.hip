@@ -234,19 +234,25 @@ struct NtProblem {
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
-// Shapes the MFMA kernel takes (pointer alignment is checked separately);
-// everything else goes to the any-shape kernel.
+size_t ksteps_of(const NtProblem &q) { return (q.Kbytes + 127) / 128; }      // the last one may be partial
+
+// Shapes the MFMA kernel takes (pointer alignment is checked separately); everything else goes to the any-shape
+// kernel.  K is a whole number of 16-byte chunks (the unit of a copy); a last K step of fewer than 128 bytes is
+// filled up with zeros on the way into LDS (GemmArgs::k_tail), which the reference's dispatch covers with its
+// 64- and 32-wide K tiles (hip_mix_gemm_kernel.cpp:442-463).
 bool mfma_shape_ok(const NtProblem &q) {
     const size_t es = (q.arith == AR_BF16 || q.arith == AR_F16) ? 2 : 1, krows = q.Kbytes / es;
     // 32-bit buffer offsets: 256 tile rows of a K-contiguous operand (plus the 3072 bytes by which the solo kernels
-    // shift their descriptors), every k row of a K-major one
+    // shift their descriptors), every k row of a K-major one.  With a partial last K step the lanes past the end of
+    // a row mark their offsets with bit 31: every valid offset then has to stay below 2^31.
+    const size_t lim = (size_t)1 << (q.Kbytes % 128 ? 31 : 32);
     const bool a_ok = (q.kmaj & 1) ? (krows * q.lda_bytes < ((size_t)1 << 32) && q.lda_bytes >= q.M * es)
-                                   : q.lda_bytes * 256 + 4096 < ((size_t)1 << 32);
+                                   : q.lda_bytes * 256 + 4096 < lim;
     const bool b_ok = (q.kmaj & 2) ? (krows * q.ldb_bytes < ((size_t)1 << 32) && q.ldb_bytes >= q.N * es)
-                                   : q.ldb_bytes * 256 + 4096 < ((size_t)1 << 32);
+                                   : q.ldb_bytes * 256 + 4096 < lim;
     // block scales: the kernel addresses a_scale with 32-bit byte offsets ((kb * as_ks + m) * 4)
     const bool s_ok = !q.block || ((q.Kbytes + 127) / 128) * std::max<size_t>(q.M, q.as_ks) * 4 < ((size_t)1 << 32);
-    return q.Kbytes % 128 == 0 && q.Kbytes > 0 && q.lda_bytes % 16 == 0 && q.ldb_bytes % 16 == 0 && a_ok && b_ok && s_ok &&
+    return q.Kbytes % 16 == 0 && q.Kbytes > 0 && q.lda_bytes % 16 == 0 && q.ldb_bytes % 16 == 0 && a_ok && b_ok && s_ok &&
            q.M < ((size_t)1 << 31) && q.N < ((size_t)1 << 31) && q.ldc < ((size_t)1 << 32);
 }
 
@@ -468,7 +474,7 @@ bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes
     if (!tab || !tab_km) return false;
     if (forced()) return row_by_name(tab_km, count_km, g_ctx.force_config) >= 0;   // a forced row: as stored where the K-major family has it
     if (g_ctx.kmajor == 2) return true;                                        // measurements: as stored wherever possible
-    const size_t ksteps = q.Kbytes / 128;
+    const size_t ksteps = ksteps_of(q);
     const bool may_split = q.split_k == 0;
     uint32_t ns = 0;
     double t_km = 0, t_nt = 8.0;                    // a skinny K-contiguous launch: about 8 us
@@ -525,14 +531,14 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
     const Variant *tab = table_for(q.arith, q.block, q.kmaj, &count);
     if (!tab) return QGEMM_ERR_UNSUPPORTED;
     uint32_t model_split = 0;
-    int vi = choose_variant(tab, count, q.M, q.N, q.Kbytes / 128, q.block, q.kmaj, g_ctx.num_cus, q.split_k == 0, &model_split);
+    int vi = choose_variant(tab, count, q.M, q.N, ksteps_of(q), q.block, q.kmaj, g_ctx.num_cus, q.split_k == 0, &model_split);
     if (may_split_rows && vi >= 0 && !forced() && g_ctx.force_split <= 0 && q.split_k == 0 && model_split <= 1 &&
         q.M > 128 && q.kmaj == 0) {
         uint32_t ns = 0;
         double t_single = 0;
-        const int ci = choose_by_cost(tab, count, q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, false, &ns, &t_single);
+        const int ci = choose_by_cost(tab, count, q.M, q.N, ksteps_of(q), q.block, g_ctx.num_cus, false, &ns, &t_single);
         if (ci >= 0 && tab[ci].bm == tab[vi].bm && tab[ci].bn == tab[vi].bn && tab[ci].kgroups == tab[vi].kgroups) {
-            const size_t m_main = rows_for_full_rounds(tab, count, q.M, q.N, q.Kbytes / 128, q.block, g_ctx.num_cus, t_single);
+            const size_t m_main = rows_for_full_rounds(tab, count, q.M, q.N, ksteps_of(q), q.block, g_ctx.num_cus, t_single);
             if (m_main) {
                 NtProblem q_main = q, q_rest = q;
                 q_main.M = m_main;
@@ -561,7 +567,8 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
     a.bs = q.bs;
     a.M = (uint32_t)q.M;
     a.N = (uint32_t)q.N;
-    a.ksteps = (uint32_t)(q.Kbytes / 128);
+    a.ksteps = (uint32_t)ksteps_of(q);
+    a.k_tail = (uint32_t)(q.Kbytes % 128);
     a.lda = (uint32_t)q.lda_bytes;
     a.ldb = (uint32_t)q.ldb_bytes;
     a.tiles_m = (uint32_t)((q.M + v.bm - 1) / v.bm);

@@ -169,8 +169,13 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_BF16, 0, 2, 1024, 1024, 1024) == "64x128_w1x4_k2_nn"
     assert plan(Q.DT_BF16, 0, 2, 8192, 8192, 8192) == "transpose+256x256_w2x2_solo"
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 2, 1024, 1024, 1024).startswith("transpose+")   # no K-major int8 family
-    # K not a multiple of 128 bytes: the any-shape kernel
+    # K bytes not a multiple of 16: the any-shape kernel; whole 16-byte chunks with a partial last K step: the MFMA kernels
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 100, 100, 100) == "strided_any_shape"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7200) == "256x256_w2x4_solo8"       # (57 K blocks: no twin)
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7216) == "256x256_w2x4_solo8"
+    assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4000) == plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4096)
+    assert plan(Q.DT_BF16, 0, 0, 1024, 1024, 1000) == plan(Q.DT_BF16, 0, 0, 1024, 1024, 1024)
+    assert plan(Q.DT_BF16, 0, 0, 1024, 1024, 1004) == "strided_any_shape"
     # forced rows are honoured, and a forced split shows in the name
     Q.force_config("128x128_w2x2_dma")
     Q.set_option("force_split", 4)

@@ -126,6 +126,39 @@ def test_cfg4_fp8_block_scaled_6144x4608x7168():
         assert_close(got[:, sel], ref, what=f"{Q.last_config()} cols of block {nb}")
 
 
+def test_cfg4_shape_with_k_7200_stays_on_the_matrix_cores():
+    """Config 4's shape with K = 7200 (56 whole K blocks and a quarter of one; K % 32 == 0 is all the reference's
+    dispatch asks for, hip_mix_gemm_kernel.cpp:442-463), in both storages: the pipelined MFMA kernels, not the any-shape
+    kernel; oracle on 16 full rows and the columns of one 128-block."""
+    M, N, K = 6144, 4608, 7200
+    say("cfg4 shape, K = 7200")
+    KB = (K + 127) // 128
+    assert Q.plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, M, N, K).startswith("256x256_w2x4_solo8")
+    assert "strided" not in Q.plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, M, N, K)
+    qa, _ = R.quantize_fp8(R.fill_normal((M, K), 42))
+    qb, _ = R.quantize_fp8(R.fill_normal((N, K), 43))
+    as_ = R.fill_uniform((M, KB), 44, 0.5, 2.0) * np.float32(5.0 / 448.0)
+    bs = R.fill_uniform((N // 128, KB), 45, 0.5, 2.0) * np.float32(5.0 / 448.0)
+    c = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
+    name = Q.last_config()
+    assert name.startswith("256x256_w2x4_solo8"), name
+    got = host(c)
+    rows = _sample(M, 16, 5)
+    fb = R.decode_fp8(qb)
+    assert_close(got[rows], R.gemm_fp8_block(R.decode_fp8(qa[rows]), fb, as_[rows], bs), what=name)
+    del fb
+    nb = 17
+    sel = np.arange(nb * 128, nb * 128 + 128, 9)
+    assert_close(got[:, sel], R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb[sel]), as_, bs[nb:nb + 1]), what=name + " cols")
+    # the reference's storage: A is K x M, B is K x N, scales K-block-major
+    c2 = torch.zeros_like(c)
+    Q.fp8_mm(fp8_tensor(np.ascontiguousarray(qa.T)).t(), fp8_tensor(np.ascontiguousarray(qb.T)).t(),
+             dev(np.ascontiguousarray(as_.T)).t(), dev(np.ascontiguousarray(bs.T)).t(), c2)
+    assert "strided" not in Q.last_config(), Q.last_config()
+    assert_close(host(c2)[rows], got[rows], rtol=2.0 ** -7, atol=1e-3, what="reference storage against K-contiguous")
+
+
 @pytest.mark.parametrize("M", [16, 64, 128])
 def test_cfg5_skinny_split_k(M):
     """Skinny M, N=7168, K=2048, int8 (bit-exact) and fp8 (tolerance) with per-matrix scales; whole matrix.

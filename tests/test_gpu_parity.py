@@ -296,8 +296,8 @@ def test_fp8_mm_dispatch_errors_like_the_reference():
         assert e.value.status == status and "not divisible" in str(e.value)
 
 
-@pytest.mark.parametrize("shape", [(64, 64, 96), (32, 96, 160), (33, 17, 50)])
-def test_any_shape_kernel_k_not_multiple_of_128(shape):
+@pytest.mark.parametrize("shape", [(64, 64, 100), (32, 96, 168), (33, 17, 50)])
+def test_any_shape_kernel_k_not_multiple_of_16(shape):
     M, N, K = shape
     say("any-shape", shape)
     qa, sa, qb, sb = int8_inputs(M, N, K, seed=41)
@@ -306,7 +306,7 @@ def test_any_shape_kernel_k_not_multiple_of_128(shape):
     assert Q.last_config() == "strided_any_shape"
     assert np.array_equal(host(c), R.gemm_i8_i32(qa, qb))
     qa, sa, qb, sb = fp8_inputs(M, N, K, seed=42)
-    if K % 32 == 0 and M % 32 == 0 and N % 32 == 0:
+    if M % 32 == 0 and N % 32 == 0:
         as_ = R.fill_uniform((M, (K + 127) // 128), 43, 0.5, 2.0) / np.float32(448)
         bs = R.fill_uniform(((N + 127) // 128, (K + 127) // 128), 44, 0.5, 2.0) / np.float32(448)
         ref = R.gemm_fp8_block(R.decode_fp8(qa), R.decode_fp8(qb), as_, bs)      # bk by the reference's dispatch
