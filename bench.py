@@ -232,8 +232,49 @@ def one_shape(Q, torch, dev, spec, launches):
     e0.record(); g.replay(); e1.record()
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / launches
-    return {"type": fam, "M": M, "N": N, "K": K, "kernel": Q.last_config(), "launches": launches, "us_per_launch": round(us, 2),
-            "tflops": round(2.0 * M * N * K / us / 1e6, 1)}
+    out = {"type": fam, "M": M, "N": N, "K": K, "kernel": Q.last_config(), "launches": launches, "us_per_launch": round(us, 2),
+           "tflops": round(2.0 * M * N * K / us / 1e6, 1)}
+    # With the measurement build of the library (QGEMM_LIBRARY=qgemm_amd/libqgemm_dbg.so, `make DEBUG=1`): the time
+    # stamps gemm_nt_kernel takes per wave (start, K loop entered, K loop left, end; a 100 MHz clock all CUs share) of
+    # one eager launch that follows twenty untimed ones, summarised per round of workgroups (CUs at a time).
+    try:
+        Q.set_option("dbg_ptr", 0)
+    except Q.QgemmError:
+        return out
+    if "+" in out["kernel"] or "skinny" in out["kernel"] or "splitk" in out["kernel"]:
+        return out
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    slots = 1 << 16                                          # workgroups x waves of any variant on any shape tried here
+    buf = torch.zeros(slots * 4, dtype=torch.int64, device=dev)
+    Q.set_option("dbg_ptr", buf.data_ptr())
+    for _ in range(20):
+        fn()
+    buf.zero_()
+    torch.cuda.synchronize()
+    fn()
+    torch.cuda.synchronize()
+    Q.set_option("dbg_ptr", 0)
+    t = buf.view(slots, 4).double() * 10.0                   # ticks -> ns
+    used = t[:, 3] > 0
+    n_waves = int(used.sum())
+    t = t[:n_waves]
+    t0 = float(t[:, 0].min())
+    # stamps of a workgroup = those of its first wave
+    nw = 8 if "w2x4" in out["kernel"] or "w1x4_k2" in out["kernel"] else 4
+    nw = {"128x128_w2x2_k2": 12, "64x128_w1x4_k2": 12, "256x128_w2x2_cw": 8, "256x128_w2x2_cw_ks": 8}.get(out["kernel"].replace("_tn", "").replace("_nn", ""), nw)
+    w = t[::nw]
+    n_wg = w.shape[0]
+    rounds = []
+    for r0 in range(0, n_wg, cus):
+        g = w[r0:r0 + cus]
+        rounds.append({"workgroups": int(g.shape[0]), "start_us": round(float(g[:, 0].mean() - t0) / 1e3, 2),
+                       "to_k_loop_us": round(float((g[:, 1] - g[:, 0]).mean()) / 1e3, 2),
+                       "k_loop_us": round(float((g[:, 2] - g[:, 1]).mean()) / 1e3, 2),
+                       "us_per_k_step": round(float((g[:, 2] - g[:, 1]).mean()) / 1e3 / ((K * (2 if fam in ("bf16", "fp16") else 1) + 127) // 128), 3),
+                       "epilogue_us": round(float((g[:, 3] - g[:, 2]).mean()) / 1e3, 2),
+                       "end_us_mean": round(float(g[:, 3].mean() - t0) / 1e3, 2), "end_us_last": round(float(g[:, 3].max() - t0) / 1e3, 2)})
+    out["stamps"] = {"waves": n_waves, "workgroups": n_wg, "waves_per_workgroup": nw, "rounds_of_%d_CUs" % cus: rounds}
+    return out
 
 
 STREAM_SHAPES = [(1, 8192, 8192), (16, 4096, 4096), (16, 4096, 14336), (64, 4096, 14336), (16, 8192, 8192), (64, 8192, 8192),

@@ -63,7 +63,8 @@ struct Context {
     long as_groups = 1;         // 0: a_scale always one K block per copy on the rows with two K groups (see run_nt)
     long k_rot = -1;            // -1: rotated K start for at most 256 rows (see plan_nt), 0: never, n: steps per column tile
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
-    long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch
+    long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch;
+                                // 2: always where the geometry allows it, whatever the estimate says (for measurements)
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes; 2: never
                                 // where a K-major kernel fits the shape (for measurements and tests)
     std::string last_config;
@@ -523,6 +524,7 @@ size_t rows_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, s
     } else {
         t_rest = 5.0 + (double)N * ksteps * 128.0 / 4.0e6;      // B streamed once, about 4 TB/s
     }
+    if (g_ctx.row_split == 2) return m_main;
     return t_main + t_rest + 6.0 < 0.97 * t_single ? m_main : 0;
 }
 
