@@ -58,7 +58,7 @@ constexpr bool kmajor_can(int bm, int bn, int nw) {
 
 template <class C>
 static Variant gemm_row(const char *name, bool auto_ok) {
-    return Variant{name, C::ARITH, C::BLOCK_SCALE, C::BM, C::BN, C::THREADS, C::LDS_BYTES, auto_ok, C::KG, C::ASK,
+    return Variant{name, C::ARITH, C::BLOCK_SCALE, C::BM, C::BN, C::THREADS, C::LDS_BYTES, auto_ok, C::COPYW, C::KG, C::ASK,
                    C::AS_ANY_STRIDE, -1, 0, &launch_variant<C>};
 }
 // row of the skinny-M kernel (gemm_skinny.cuh): 16 * TM rows x 16 * TN columns, eight waves splitting K between them.
@@ -66,7 +66,7 @@ static Variant gemm_row(const char *name, bool auto_ok) {
 template <int TM, int TN = 2>
 static Variant skinny_row(const char *name) {
     using C = SkinnyCfg<INST_ARITH, TM, kBlock, TN>;
-    return Variant{name, C::ARITH, C::BLOCK_SCALE, C::BM, C::BN, C::THREADS, C::LDS_BYTES, false, 8, false, C::BLOCK_SCALE,
+    return Variant{name, C::ARITH, C::BLOCK_SCALE, C::BM, C::BN, C::THREADS, C::LDS_BYTES, false, false, 8, false, C::BLOCK_SCALE,
                    -1, 0, &launch_skinny<C>};
 }
 

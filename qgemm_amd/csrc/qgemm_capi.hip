@@ -334,6 +334,8 @@ int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t kst
 
 int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
                 bool may_split, uint32_t *nsplit_out);
+size_t rows_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus,
+                            double t_single, double *t_split = nullptr);
 
 // The skinny-M kernel (gemm_skinny.cuh: the K split inside the workgroup, eight waves each on every eighth K step)
 // takes over from the narrow simple-pipeline tiles where it is faster: one row tile (M <= 128), a strip of 32
@@ -459,11 +461,18 @@ int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps
 }
 
 // Should the problem run with these operands read K-major, as they are stored (strides between k rows given)?
-// Yes when the shape fits and the estimate for the K-major family (simple pipeline, two stages, transposing reads:
-// 15 % on top of the estimate) beats the K-contiguous kernel plus the transpose launches in front of it (4 us per
-// operand and the matrix read and written at 5.5 TB/s; block scales 2048^3 in the reference's layout: 23.3 us as
-// stored, 29.3 us behind two transposes; 1024 x 4096 x 4096: 39.9 against 37.2).  Large shapes keep the transposes
-// and the pipelined 256 x 256 tile; small and mid-size ones save the launches.
+// Yes when the shape fits and the estimate for the K-major family beats the K-contiguous kernel plus the transpose
+// launches in front of it (4 us per operand and the matrix read and written at 5.5 TB/s; block scales 2048^3 in the
+// reference's layout: 23.3 us as stored, 29.3 us behind two transposes; 1024 x 4096 x 4096: 39.9 against 37.2).
+// The simple-pipeline rows pay 15 % on top of the estimate for their transposing reads.  The 256 x 128 row with
+// copying waves needs per K step what its K-contiguous form needs, and is taken up to 2.5 % above the other route's
+// estimate (which counts a row split where the K-contiguous plan would make one, and runs low for one round of
+// 256 x 256 tiles behind transposes).  Measured, as stored against through the transposes, us: fp8_mm 4096^3
+// 65.3 / 73.9, 2048 x 4096 x 4096 35.0 / 46.9, 3072 x 8192 x 4096 102.8 / 110.4, bf16 with B stored K x N 4096^3
+// 101.4 / 109.6, 2048 x 8192 x 8192 194.6 / 223.3, 2048 x 4096 x 4096 52.2 / 68.2; the largest shapes keep the
+// transposes and the 256 x 256 tile: config 4 in the reference's storage 207.8 / 194.6, 8192^3 506.6 / 465.2 (fp8_mm)
+// and 786.0 / 742.4 (bf16), 6144^3 240.3 / 229.6 and 356.7 / 348.6.  Over 19 shapes the ratio of the two estimates is
+// within 4 % of the measured ratio on 15 and the choice is the faster route on all but bf16 3072 x 4096 x 4096 (4 %).
 bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes) {
     if (!g_ctx.kmajor) return false;
     q.kmaj = kmaj;
@@ -479,14 +488,22 @@ bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes
     const bool may_split = q.split_k == 0;
     uint32_t ns = 0;
     double t_km = 0, t_nt = 8.0;                    // a skinny K-contiguous launch: about 8 us
-    if (choose_by_cost(tab_km, count_km, q.M, q.N, ksteps, q.block, g_ctx.num_cus, may_split, &ns, &t_km) < 0) return false;
+    const int vk = choose_by_cost(tab_km, count_km, q.M, q.N, ksteps, q.block, g_ctx.num_cus, may_split, &ns, &t_km);
+    if (vk < 0) return false;
     if (q.M > 128 && choose_by_cost(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, may_split, &ns, &t_nt) < 0)
         return false;
+    if (q.M > 128 && may_split) {                    // (the K-contiguous route may split the rows into two launches)
+        double t_single = 0, t_split = 0;
+        uint32_t ns1 = 0;
+        if (choose_by_cost(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, false, &ns1, &t_single) >= 0 &&
+            rows_for_full_rounds(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, t_single, &t_split) && t_split < t_nt)
+            t_nt = t_split;
+    }
     const double kbytes = (double)q.Kbytes;         // K * element size
     t_nt += 1.0;                                     // a transpose launch per operand: 4 us and the matrix read and written
     if (kmaj & 1) t_nt += 4.0 + 2.0 * (double)q.M * kbytes / 5.5e6;
     if (kmaj & 2) t_nt += 4.0 + 2.0 * (double)q.N * kbytes / 5.5e6;
-    return 1.15 * t_km <= t_nt;
+    return tab_km[vk].copy_waves ? t_km <= 1.025 * t_nt : 1.15 * t_km <= t_nt;
 }
 
 struct Plan {
@@ -509,7 +526,7 @@ struct Plan {
 // skinny-M kernel).  Returns 0 for "do not split": when the estimate of the two launches (plus 6 us for the
 // second) is not at least 3 % below the estimate t_single of the one.
 size_t rows_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus,
-                            double t_single) {
+                            double t_single, double *t_split) {
     if (!g_ctx.row_split) return 0;
     const size_t tn = (N + 255) / 256, tiles = ((M + 255) / 256) * tn, full = tiles / cus;
     if (full == 0 || tiles % cus == 0) return 0;
@@ -524,6 +541,7 @@ size_t rows_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, s
     } else {
         t_rest = 5.0 + (double)N * ksteps * 128.0 / 4.0e6;      // B streamed once, about 4 TB/s
     }
+    if (t_split) *t_split = t_main + t_rest + 6.0;
     if (g_ctx.row_split == 2) return m_main;
     return t_main + t_rest + 6.0 < 0.97 * t_single ? m_main : 0;
 }

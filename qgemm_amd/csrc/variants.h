@@ -13,6 +13,7 @@ struct Variant {
     bool block_scale;
     int bm, bn, threads, lds_bytes;
     bool auto_ok;   // the shape heuristic may pick this row (the others are reachable by name, option "force_config")
+    bool copy_waves;   // solo schedule with four computing and four copying waves (GemmCfg::COPYW)
     int kgroups;    // 2: two sets of waves per workgroup, each computing every other K step (GemmCfg::KG);
                     // 8: the skinny-M kernel, eight waves each computing every eighth K step (gemm_skinny.cuh)
     bool a_scale_k_contiguous;   // block scales: the kernel reads a_scale[m * ld + kb] as QGEMM_LAYOUT_K_CONTIGUOUS passes

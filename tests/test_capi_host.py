@@ -168,6 +168,9 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 6144, 4608, 7168) == "transpose+256x256_w2x4_solo8"
     assert plan(Q.DT_BF16, 0, 2, 1024, 1024, 1024) == "64x128_w1x4_k2_nn"
     assert plan(Q.DT_BF16, 0, 2, 8192, 8192, 8192) == "transpose+256x256_w2x2_solo"
+    # large shapes whose transposes are a sizeable part: as stored, on the K-major 256 x 128 row with copying waves
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 4096, 4096, 4096) == "256x128_w2x2_cw_tn"
+    assert plan(Q.DT_BF16, 0, 2, 2048, 8192, 8192) == "256x128_w2x2_cw_nn"
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 2, 1024, 1024, 1024).startswith("transpose+")   # no K-major int8 family
     # K bytes not a multiple of 16: the any-shape kernel; whole 16-byte chunks with a partial last K step: the MFMA kernels
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 100, 100, 100) == "strided_any_shape"
