@@ -209,8 +209,10 @@ def one_shape(Q, torch, dev, spec, launches):
         KB = (K + 127) // 128
         sa = (torch.rand(M, KB, device=dev) + 0.5) / 448; sb = (torch.rand((N + 127) // 128, KB, device=dev) + 0.5) / 448
         fn = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_BLOCK128)
-    elif fam == "int8":
+    elif fam in ("int8", "int8f32"):                        # int8: bf16 out; int8f32: fp32 out (config 2's output type)
         a, sa = _quant_i8(torch.randn(M, K, device=dev)); b, sb = _quant_i8(torch.randn(N, K, device=dev))
+        if fam == "int8f32":
+            c = torch.empty(M, N, dtype=torch.float32, device=dev)
         fn = lambda: Q.int8_mm(a, b, sa, sb, c)
     elif fam in ("bf16", "fp16"):
         dt = torch.bfloat16 if fam == "bf16" else torch.float16
@@ -218,7 +220,7 @@ def one_shape(Q, torch, dev, spec, launches):
         c = torch.empty(M, N, dtype=dt, device=dev)
         fn = lambda: Q.gemm(a, b, c, "nk")
     else:
-        raise SystemExit("bench.py --shape: type must be fp8, fp8block, int8, bf16 or fp16")
+        raise SystemExit("bench.py --shape: type must be fp8, fp8block, int8, int8f32, bf16 or fp16")
     for _ in range(3):
         fn()
     torch.cuda.synchronize()
@@ -271,6 +273,7 @@ def one_shape(Q, torch, dev, spec, launches):
                        "to_k_loop_us": round(float((g[:, 1] - g[:, 0]).mean()) / 1e3, 2),
                        "k_loop_us": round(float((g[:, 2] - g[:, 1]).mean()) / 1e3, 2),
                        "us_per_k_step": round(float((g[:, 2] - g[:, 1]).mean()) / 1e3 / ((K * (2 if fam in ("bf16", "fp16") else 1) + 127) // 128), 3),
+                       "k_loop_end_us": round(float(g[:, 2].mean() - t0) / 1e3, 2),
                        "epilogue_us": round(float((g[:, 3] - g[:, 2]).mean()) / 1e3, 2),
                        "end_us_mean": round(float(g[:, 3].mean() - t0) / 1e3, 2), "end_us_last": round(float(g[:, 3].max() - t0) / 1e3, 2)})
     out["stamps"] = {"waves": n_waves, "workgroups": n_wg, "waves_per_workgroup": nw, "rounds_of_%d_CUs" % cus: rounds}
@@ -431,7 +434,7 @@ def main():
                     help="only time 160 ... 3072 rows against six weight shapes, this library and the vendor library from "
                          "replayed graphs, print one JSON line and exit")
     ap.add_argument("--shape", default="",
-                    help="only run this library on one shape, e.g. fp8:2048x2048x8192 (fp8 | fp8block | int8 | bf16 | fp16), "
+                    help="only run this library on one shape, e.g. fp8:2048x2048x8192 (fp8 | fp8block | int8 | int8f32 | bf16 | fp16), "
                          "--steps launches from a replayed graph; print one JSON line and exit")
     ap.add_argument("--skinny-probe", action="store_true",
                     help="only probe where the skinny-M kernel (config 5) spends its time, print one JSON line and exit")

@@ -70,7 +70,8 @@ struct GemmArgs {
     int per_matrix_scale; // multiply by as[0]*bs[0] in the epilogue
     int vec_store;        // 0: scalar stores; 1: C and ldc allow 4-element vector stores; 2: also 16-byte row pieces
     uint32_t k_rot;                  // simple pipeline and skinny-M kernel: the workgroups of column tile i start their K loops (i * k_rot) % nk steps in (0: at 0)
-    uint32_t stagger, stagger_wgs;   // the first stagger_wgs workgroups start (id / 8 % 4) * stagger microseconds late (0: off)
+    uint32_t stagger, stagger_wgs;   // the first stagger_wgs workgroups start (id / 8 % stagger_groups) * stagger microseconds late (0: off)
+    uint32_t stagger_groups;
     unsigned long long *dbg_cycles;   // measurement builds only (QGEMM_STAMP): time stamps per wave
 };
 
@@ -290,13 +291,15 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
     QGEMM_STAMP(0);
 
     // Staggered start (the host asks for it where C is written in 4-byte elements over three or more rounds of
-    // tiles).  Left alone, all CUs finish a round of 256 x 256 tiles together and write 64 MiB of C at once: the
-    // epilogue of such a tile takes 10 - 12 us against 4.6 us for the 2-byte output, with the matrix cores of the
-    // whole part idle.  The workgroups of the first round therefore start in four groups about 2 us apart (s_sleep:
-    // 64 clocks per unit), the offsets carry through every later round, and the bursts interleave with other CUs'
-    // K loops: int8 8192^3 to f32 397 -> 386 us, 8192 x 8192 x 4096 232 -> 223 us (interleaved A/B in one process).
+    // tiles).  Left alone, all CUs finish a round of 256 x 256 tiles together and write 64 MiB of C at once, which is
+    // what the memory takes 10 us to absorb: the epilogue of such a tile takes 10 - 12 us against 4.6 us for the 2-byte
+    // output, with the matrix cores of the whole part idle.  The workgroups of the first round therefore start in
+    // groups a microsecond or two apart (s_sleep: 64 clocks per unit), the offsets carry through every later round,
+    // and the bursts interleave with other CUs' K loops.  int8 8192^3 to f32, interleaved in one process, us: none
+    // 381.0, four groups 2 us apart 374.2, eight groups 1 us apart 367.9 (what the host asks for), 8 x 2 371.7,
+    // 16 x 1 383.6, 32 x 1 412.3; the same product with bf16 output 359.9.  8192 x 8192 x 4096: 226.4 / 216.2 / 213.2.
     if (p.stagger > 0 && blockIdx.x < p.stagger_wgs) {
-        const int g = (blockIdx.x >> 3) & 3;            // (workgroup i runs on XCD i % 8: whole rows of XCDs per group)
+        const int g = (blockIdx.x >> 3) % p.stagger_groups;            // (workgroup i runs on XCD i % 8: whole rows of XCDs per group)
         for (int i = 0; i < g * (int)p.stagger; ++i) __builtin_amdgcn_s_sleep(32);
     }
     const int tid = threadIdx.x;

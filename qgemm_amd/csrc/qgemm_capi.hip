@@ -63,6 +63,7 @@ struct Context {
     long as_groups = 1;         // 0: a_scale always one K block per copy on the rows with two K groups (see run_nt)
     long k_rot = -1;            // -1: rotated K start for at most 256 rows (see plan_nt), 0: never, n: steps per column tile
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
+    long stagger_groups = 8;    // groups the workgroups of the first round start in
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch;
                                 // 2: always where the geometry allows it, whatever the estimate says (for measurements)
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes; 2: never
@@ -684,8 +685,9 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
         // (with fewer than 32 K steps the offsets are too large a part of a tile's time: 7000 x 7168 x 2048 int8 to
         // f32 128 us without, 139 us with)
         const bool spread = v.bm == 256 && v.bn == 256 && ob == 4 && pl.tiles >= 3 * (size_t)g_ctx.num_cus && a.ksteps >= 32;
-        a.stagger = g_ctx.stagger >= 0 ? (uint32_t)g_ctx.stagger : (spread ? 2u : 0u);
+        a.stagger = g_ctx.stagger >= 0 ? (uint32_t)g_ctx.stagger : (spread ? 1u : 0u);
         a.stagger_wgs = (uint32_t)g_ctx.num_cus;
+        a.stagger_groups = (uint32_t)std::max<long>(1, std::min<long>(32, g_ctx.stagger_groups));
         hipError_t e = v.launch(a, (uint32_t)pl.tiles, stream);
         g_ctx.last_config = std::string(v.name) + kmaj_suffix(q.kmaj);
         return e == hipSuccess ? QGEMM_OK : QGEMM_ERR_LAUNCH;
@@ -970,6 +972,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "group_m")) g_ctx.force_group_m = value;
     else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
     else if (!std::strcmp(key, "stagger")) g_ctx.stagger = value;
+    else if (!std::strcmp(key, "stagger_groups")) g_ctx.stagger_groups = value;
     else if (!std::strcmp(key, "k_rot")) g_ctx.k_rot = value;
     else if (!std::strcmp(key, "as_groups")) g_ctx.as_groups = value;
 #if QGEMM_DEBUG_BUILD
