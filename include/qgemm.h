@@ -90,9 +90,12 @@ int qgemm_gemm(int in_dtype, int out_dtype, int layout_b, const void *A, size_t 
  * Replaces select_BLOCK_TILE_SIZE_M / fp8_mm (src/mix_gemm/hip_mix_gemm_kernel.cpp:489-516)
  * and the int8_mm stub (src/gemm/sm80_gemm_kernel.cu:14-22).
  *   in_dtype   I8 (int32 accumulate, exact) | F8E4M3 (fp32 accumulate)
- *   out_dtype  F32 | BF16 | F16 ; I32 with I8 input returns the raw accumulators (scales ignored)
+ *   out_dtype  F32 | BF16 | F16 ; I32 with I8 input and per-matrix scales returns the raw accumulators (scales ignored)
  *   scale_mode PER_MATRIX: C = acc * (a_scale[0] * b_scale[0])
- *              BLOCK128  : acc += (P_kb * a_scale[m,kb]) * b_scale[n/128,kb] per 128-wide K block
+ *              BLOCK128  : acc += (P_kb * a_scale[m,kb]) * b_scale[n/128,kb] per 128-wide K block (the last block may
+ *                          be partial); P_kb is the fp32 partial of an fp8 block or the exact int32 partial of an int8
+ *                          block, converted to fp32 once (the int8 twin of hip_mix_gemm_kernel.cpp:231-244, which the
+ *                          reference only has for fp8)
  *   layout     see qgemm_layout_t;  C is row-major with leading dimension ldC
  *   split_k    0 = choose, 1 = never split, n > 1 = split K into n slices (deterministic
  *              two-pass reduction through the library workspace)
@@ -139,7 +142,7 @@ int qgemm_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t 
  *   x        rows x cols, F32 / BF16 / F16, row stride ld elements (device)
  *   q        rows x cols bytes (I8 or F8E4M3), row stride ldq
  *   scales   QGEMM_QUANT_PER_MATRIX: 1 float, s = max|x| / 127 (int8) or / 448 (fp8)
- *            QGEMM_QUANT_BLOCK_1x128 / _128x128 (fp8 only): one float per block, written to
+ *            QGEMM_QUANT_BLOCK_1x128 / _128x128: one float per block (max|x| of the block / 127 or / 448), written to
  *            scales[ib * scale_rs + jb * scale_cs] (ib: block row, jb: block column; strides in floats),
  *            so the a_scale / b_scale arrangement of either layout of qgemm_scaled_gemm can be produced
  *            directly (hip_mix_gemm_kernel.cpp:137,149)

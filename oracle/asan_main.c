@@ -31,6 +31,7 @@ float ref_amax(const float *, size_t);
 float ref_quantize_int8(const float *, int8_t *, size_t);
 float ref_quantize_fp8(const float *, uint8_t *, size_t);
 void ref_quantize_fp8_block(const float *, uint8_t *, float *, size_t, size_t, size_t, size_t);
+void ref_quantize_int8_block(const float *, int8_t *, float *, size_t, size_t, size_t, size_t);
 void ref_transpose(const void *, void *, size_t, size_t, size_t);
 void ref_gemm_i8_i32(const int8_t *, size_t, size_t, const int8_t *, size_t, size_t, int32_t *, size_t, size_t, size_t, size_t);
 void ref_scale_i32_to_f32(const int32_t *, float *, size_t, float, float);
@@ -40,6 +41,8 @@ void ref_gemm_fp8_block(const float *, size_t, size_t, const float *, size_t, si
                         const float *, size_t, size_t, float *, size_t, size_t, size_t, size_t, size_t);
 void ref_gemm_fp8_block_f64(const float *, size_t, size_t, const float *, size_t, size_t, const float *, size_t, size_t,
                             const float *, size_t, size_t, double *, size_t, size_t, size_t, size_t);
+void ref_gemm_i8_block(const int8_t *, size_t, size_t, const int8_t *, size_t, size_t, const float *, size_t, size_t,
+                       const float *, size_t, size_t, float *, size_t, size_t, size_t, size_t);
 size_t ref_select_tile(size_t, int);
 void ref_block_swizzle(size_t, size_t, size_t, size_t, size_t *, size_t *);
 double ref_max_abs_diff(const float *, const float *, size_t);
@@ -121,7 +124,14 @@ static void check_quantizers(void) {
                 const float s = sc[(r / br) * nbc + c / 128];
                 CHECK(fabsf(xs[r * cols + c] - s * ref_fp8_e4m3_to_f32(q[r * cols + c])) <= 0.0626f * fabsf(xs[r * cols + c]) + 0.002f * s);
             }
-        free(xs); free(q); free(sc);
+        int8_t *q8 = xmalloc(rows * cols);
+        ref_quantize_int8_block(xs, q8, sc, rows, cols, br, 128);
+        for (size_t r = 0; r < rows; ++r)
+            for (size_t c = 0; c < cols; ++c) {
+                const float s = sc[(r / br) * nbc + c / 128];
+                CHECK(fabsf(xs[r * cols + c] - s * (float)q8[r * cols + c]) <= 0.5001f * s);
+            }
+        free(xs); free(q); free(q8); free(sc);
     }
     free(x); free(qi); free(qf);
 }
@@ -198,6 +208,19 @@ static void check_gemms(void) {
                                        bs[(n / 128) * bs_ns + (k / 128) * bs_ks];
                             CHECK(Cd[m * ldc + n] == acc && Cf[m * ldc + n] == (float)acc);     /* powers of two: exact */
                         }
+                }
+                /* the int8 twin: exact int32 partial per K block, power-of-two scales: exact */
+                for (size_t i = 0; i < M * ldc; ++i) Cf[i] = -9.0f;
+                ref_gemm_i8_block(Ai, a_rs, a_cs, Bi, b_ns, b_ks, as, as_ms, as_ks, bs, bs_ns, bs_ks, Cf, ldc, M, N, K);
+                for (size_t m = 0; m < M; ++m) {
+                    for (size_t n = 0; n < N; ++n) {
+                        double acc = 0;
+                        for (size_t k = 0; k < K; ++k)
+                            acc += (double)Ai[m * a_rs + k * a_cs] * Bi[n * b_ns + k * b_ks] * as[m * as_ms + (k / 128) * as_ks] *
+                                   bs[(n / 128) * bs_ns + (k / 128) * bs_ks];
+                        CHECK(Cf[m * ldc + n] == (float)acc);
+                    }
+                    for (size_t n = N; n < ldc; ++n) CHECK(Cf[m * ldc + n] == -9.0f);
                 }
             }
             free(A); free(B); free(Ai); free(Bi); free(Ci); free(Cf); free(Cs); free(Cd); free(as); free(bs);

@@ -19,6 +19,9 @@
  *                        representable inputs
  *   block-scaled GEMM    reduces to per-matrix when scales are equal,
  *                        power-of-two scales commute exactly, linearity
+ *   int8 block-scaled    the int8 twin of the block-scaled kernel (defined by the task's "int8 ... 128-block
+ *                        scales", implemented nowhere in the reference): brute force in Python integers and
+ *                        floats, unit scales = the exact int32 GEMM, power-of-two scales exact
  *   transpose            numpy .T, involution
  * The reference holds no golden vectors for the FP8 block-scaled kernel
  * (no test calls it), so that function's parity is pinned only by the
@@ -266,6 +269,33 @@ REF_API void ref_quantize_fp8_block(const float *x, uint8_t *q, float *scales, s
         }
 }
 
+/* the same blocks quantised to int8: s = amax / 127 per block, q = clamp(rint(x / s)) */
+REF_API void ref_quantize_int8_block(const float *x, int8_t *q, float *scales, size_t rows, size_t cols,
+                                     size_t br, size_t bc) {
+    size_t nbr = (rows + br - 1) / br, nbc = (cols + bc - 1) / bc;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (size_t ib = 0; ib < nbr; ++ib)
+        for (size_t jb = 0; jb < nbc; ++jb) {
+            size_t r1 = (ib + 1) * br < rows ? (ib + 1) * br : rows;
+            size_t c1 = (jb + 1) * bc < cols ? (jb + 1) * bc : cols;
+            float amax = 0.0f;
+            for (size_t r = ib * br; r < r1; ++r)
+                for (size_t c = jb * bc; c < c1; ++c) {
+                    float a = fabsf(x[r * cols + c]);
+                    if (a > amax) amax = a;
+                }
+            float s = amax > 0.0f ? amax / 127.0f : 1.0f;
+            scales[ib * nbc + jb] = s;
+            for (size_t r = ib * br; r < r1; ++r)
+                for (size_t c = jb * bc; c < c1; ++c) {
+                    float v = nearbyintf(x[r * cols + c] / s);
+                    if (v > 127.0f) v = 127.0f;
+                    if (v < -127.0f) v = -127.0f;
+                    q[r * cols + c] = (int8_t)v;
+                }
+        }
+}
+
 /* ------------------------------------------------------------------ */
 /* transpose: out[n*M + m] = in[m*N + n], src/transpose/transpose.cu:42,57 */
 /* ------------------------------------------------------------------ */
@@ -388,6 +418,30 @@ REF_API void ref_gemm_fp8_block(const float *A, size_t a_rs, size_t a_cs, const 
                 for (size_t k = k0; k < k1; ++k) p += A[m * a_rs + k * a_cs] * B[n * b_ns + k * b_ks];
                 size_t kb = k0 / 128;
                 float t = p * as[m * as_ms + kb * as_ks];
+                t = t * bs[(n / 128) * bs_ns + kb * bs_ks];
+                acc += t;
+            }
+            C[m * ldc + n] = acc;
+        }
+}
+
+/* The int8 twin of the kernel above (the reference's int8 path is a stub, src/gemm/sm80_gemm_kernel.cu:14-22, and its
+ * README asks for "int8 ... quantized" inputs beside the 128-block scales of hip_mix_gemm_kernel.cpp:231-244): the
+ * partial product of one 128-wide K block is an exact int32, converted to fp32 once and folded in exactly as the
+ * fp8 kernel folds its fp32 partial: acc += (float(P) * as[m, kb]) * bs[n/128, kb]. */
+REF_API void ref_gemm_i8_block(const int8_t *A, size_t a_rs, size_t a_cs, const int8_t *B, size_t b_ns, size_t b_ks,
+                               const float *as, size_t as_ms, size_t as_ks, const float *bs, size_t bs_ns,
+                               size_t bs_ks, float *C, size_t ldc, size_t M, size_t N, size_t K) {
+#pragma omp parallel for schedule(static)
+    for (size_t m = 0; m < M; ++m)
+        for (size_t n = 0; n < N; ++n) {
+            float acc = 0.0f;
+            for (size_t k0 = 0; k0 < K; k0 += 128) {
+                size_t k1 = k0 + 128 < K ? k0 + 128 : K;
+                int32_t p = 0;
+                for (size_t k = k0; k < k1; ++k) p += (int32_t)A[m * a_rs + k * a_cs] * (int32_t)B[n * b_ns + k * b_ks];
+                size_t kb = k0 / 128;
+                float t = (float)p * as[m * as_ms + kb * as_ks];
                 t = t * bs[(n / 128) * bs_ns + kb * bs_ks];
                 acc += t;
             }

@@ -54,12 +54,14 @@ def _load():
         "ref_quantize_int8": (f32, [vp, vp, sz]),
         "ref_quantize_fp8": (f32, [vp, vp, sz]),
         "ref_quantize_fp8_block": (None, [vp, vp, vp, sz, sz, sz, sz]),
+        "ref_quantize_int8_block": (None, [vp, vp, vp, sz, sz, sz, sz]),
         "ref_transpose": (None, [vp, vp, sz, sz, sz]),
         "ref_gemm_i8_i32": (None, [vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz]),
         "ref_scale_i32_to_f32": (None, [vp, vp, sz, f32, f32]),
         "ref_gemm_f32acc": (None, [vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz]),
         "ref_gemm_f64acc": (None, [vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz]),
         "ref_gemm_fp8_block": (None, [vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz, sz]),
+        "ref_gemm_i8_block": (None, [vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz]),
         "ref_gemm_fp8_block_f64": (None, [vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz]),
         "ref_select_tile": (sz, [sz, C.c_int]),
         "ref_block_swizzle": (None, [sz, sz, sz, sz, C.POINTER(sz), C.POINTER(sz)]),
@@ -178,6 +180,15 @@ def quantize_fp8_block(x, br, bc):
     return q, s
 
 
+def quantize_int8_block(x, br, bc):
+    x = np.ascontiguousarray(x, np.float32)
+    rows, cols = x.shape
+    q = np.empty(x.shape, np.int8)
+    s = np.empty(((rows + br - 1) // br, (cols + bc - 1) // bc), np.float32)
+    lib.ref_quantize_int8_block(_p(x), _p(q), _p(s), rows, cols, br, bc)
+    return q, s
+
+
 # -------------------------------------------------------------- transpose
 def transpose(a):
     a = np.ascontiguousarray(a)
@@ -264,6 +275,19 @@ def gemm_fp8_block(A, B, as_, bs, layout="nt", scale_layout="row", bk=None):
     Cm = np.empty((M, N), np.float32)
     lib.ref_gemm_fp8_block(_p(A), ars, acs, _p(B), bns, bks, _p(as_), sms, sks, _p(bs), tns, tks,
                            _p(Cm), N, M, N, K, bk)
+    return Cm
+
+
+def gemm_i8_block(A, B, as_, bs, layout="nt", scale_layout="row"):
+    """A, B: int8.  Exact int32 partial per 128-wide K block, folded in fp32 like gemm_fp8_block.  Returns fp32."""
+    A = np.ascontiguousarray(A, np.int8)
+    B = np.ascontiguousarray(B, np.int8)
+    as_ = np.ascontiguousarray(as_, np.float32)
+    bs = np.ascontiguousarray(bs, np.float32)
+    M, N, K, ars, acs, bns, bks = _strides(layout, A, B)
+    sms, sks, tns, tks = _scale_strides(scale_layout, as_, bs, M, N, K)
+    Cm = np.empty((M, N), np.float32)
+    lib.ref_gemm_i8_block(_p(A), ars, acs, _p(B), bns, bks, _p(as_), sms, sks, _p(bs), tns, tks, _p(Cm), N, M, N, K)
     return Cm
 
 

@@ -9,6 +9,6 @@ from .ops import (  # noqa: F401
     DT_BF16, DT_F16, DT_F32, DT_F8E4M3, DT_I8, DT_I32,
     LAYOUT_K_CONTIGUOUS, LAYOUT_REFERENCE, QUANT_BLOCK_128x128, QUANT_BLOCK_1x128, QUANT_PER_MATRIX,
     SCALE_BLOCK128, SCALE_PER_MATRIX,
-    bf16_mm, fp8_mm, gemm, int8_mm, last_config, matrix_transpose, plan, quantize, scaled_gemm, selftest_layouts,
+    bf16_mm, fp8_mm, gemm, int8_mm, int8_mm_block, last_config, matrix_transpose, plan, quantize, scaled_gemm, selftest_layouts,
     force_config, set_option, tile_map, variant_names,
 )

@@ -59,9 +59,22 @@ __global__ void __launch_bounds__(256) gemm_strided_kernel(const StridedArgs p) 
     if (m >= p.M || n >= p.N) return;
     const size_t idx = (size_t)m * p.ldc + n;
     if constexpr (IN_DT == QGEMM_DT_I8) {
-        int acc = 0;
         const int8_t *a = (const int8_t *)p.A + (size_t)m * p.a_rs;
         const int8_t *b = (const int8_t *)p.B + (size_t)n * p.b_ns;
+        if (p.scale_mode == 2) {           // exact int32 partial per 128-wide K block, folded in fp32
+            float accf = 0.0f;
+            for (uint32_t k0 = 0; k0 < p.K; k0 += kScaleBlock) {
+                const uint32_t k1 = k0 + kScaleBlock < p.K ? k0 + kScaleBlock : p.K;
+                int part = 0;
+                for (uint32_t k = k0; k < k1; ++k) part += (int)a[k * p.a_cs] * (int)b[k * p.b_ks];
+                const uint32_t kb = k0 / kScaleBlock;
+                accf += ((float)part * p.as[(size_t)m * p.as_ms + (size_t)kb * p.as_ks]) *
+                        p.bs[(size_t)(n / kScaleBlock) * p.bs_ns + (size_t)kb * p.bs_ks];
+            }
+            store_out(p.C, idx, accf, p.out_dtype);
+            return;
+        }
+        int acc = 0;
         for (uint32_t k = 0; k < p.K; ++k) acc += (int)a[k * p.a_cs] * (int)b[k * p.b_ks];
         if (p.out_dtype == QGEMM_DT_I32) {
             ((int *)p.C)[idx] = acc;

@@ -164,7 +164,7 @@ struct GemmCfg {
                   "K groups: simple pipeline, at least four stages");
     static_assert(BM % (16 * WAVES_M) == 0 && BN % (16 * WAVES_N) == 0, "wave tile must be a multiple of 16");
     static_assert(NLOAD % NW == 0, "load instructions must divide evenly over the waves");
-    static_assert(!BLOCK_SCALE || ARITH == AR_F8, "block scales are defined for fp8 only");
+    static_assert(!BLOCK_SCALE || ARITH == AR_F8 || ARITH == AR_I8, "block scales: fp8 and int8 operands");
     static_assert(!BLOCK_SCALE || (128 % WN == 0 || WN % 128 == 0), "wave tile must align with 128-wide scale blocks");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS is 160 KiB per CU");
     static_assert(PIPE != PIPE_SOLO || ((NW == 4 || NW == 8) && TN >= 4 &&
@@ -286,7 +286,11 @@ template <class C>
 __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
     extern __shared__ __attribute__((aligned(1024))) char smem[];
-    typedef typename AccT<C::ARITH>::type acc_t;
+    // part_t: what one MFMA step of 128 bytes of K delivers (int32 for int8 operands, else fp32); acc_t: the running
+    // sums.  With block scales the sums are fp32 whatever the operands: an int8 partial product of one K block is an
+    // exact int32, converted once and folded in like the fp8 kernel's fp32 partial.
+    typedef typename AccT<C::ARITH>::type part_t;
+    typedef std::conditional_t<C::BLOCK_SCALE, v4f, part_t> acc_t;
     QGEMM_STAMP_DECL(4);               // start, K loop start, K loop end, end
     QGEMM_STAMP(0);
 
@@ -700,7 +704,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             auto mma = [&](int a, int b, int half) {
                 if constexpr (PINNED)
                     mma128_inplace<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1], acc[a][b], half);
-                else
+                else if constexpr (!C::BLOCK_SCALE)       // (block scales: the K loop below starts every MFMA from zero)
                     acc[a][b] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1], acc[a][b]);
             };
             // The last two steps issue their copies (and the last one its scale fetch) past the end of K like
@@ -722,7 +726,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // a_scale[row] * b_scale, is made one row ahead: the cross-lane pick behind the first
                 // MFMA of row a-1, the multiply behind the second MFMA of row a, so two factors are live at a time.
                 constexpr int BEHIND = 2;      // MFMAs between a partial product and its fold
-                v4f part[BEHIND + 1];
+                part_t part[BEHIND + 1];
                 fetch_a_scales(kt + 1, par ^ 1);
                 fetch_b_scales(kt + 1);
                 // Order of the MFMAs of a step: row by row.  With copying waves (one computing wave per SIMD, four MFMAs
@@ -740,7 +744,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         const int pa = row_of_tile(i), pb = col_of_tile(i);
                         const float f = sc[pa % 2][(pb * 16) / 128];
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[i % (BEHIND + 1)][r] * f;
+                        for (int r = 0; r < 4; ++r) acc[pa][pb][r] += (float)part[i % (BEHIND + 1)][r] * f;
                     }
                 };
                 // the side instructions of a row go between its MFMAs, one at a time: a run of them in front
@@ -812,7 +816,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                             // folded into the running sum, scaled, two MFMAs later, so the four FMAs of a tile run
                             // under the MFMAs of the next two (hip_mix_gemm_kernel.cpp:231-244)
                             part[i % (BEHIND + 1)] = mma128<C::ARITH>(fbr[b][0], fbr[b][1], far[a % RING][0], far[a % RING][1],
-                                                                      v4f{0, 0, 0, 0});
+                                                                      part_t{0, 0, 0, 0});
                             side(a, b);
                             // the factor of a row is formed behind the MFMA that follows the row's first one: it is first
                             // used one MFMA later, and its register was last used (row a-2) one MFMA earlier at the latest
@@ -1103,18 +1107,18 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         for (int a = 0; a < C::TM; ++a)
 #pragma unroll
                             for (int j = 0; j < NBS; ++j) f[a][j] = as_cur[a] * bs_cur[j];
-                        v4f part[BEHIND + 1];
+                        part_t part[BEHIND + 1];
 #pragma unroll
                         for (int i = 0; i < NT + BEHIND; ++i) {
                             if (i < NT) {
                                 const int a = i % C::TM, b = i / C::TM;
-                                part[i % (BEHIND + 1)] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                                part[i % (BEHIND + 1)] = mma128<C::ARITH>(fb[b][0], fb[b][1], fa[a][0], fa[a][1], part_t{0, 0, 0, 0});
                             }
                             __builtin_amdgcn_sched_barrier(0);       // MFMA i first, the FMAs of tile i-2 under it
                             if (i >= BEHIND) {
                                 const int t = i - BEHIND, pa = t % C::TM, pb = t / C::TM;
 #pragma unroll
-                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[t % (BEHIND + 1)][r] * f[pa][(pb * 16) / 128];
+                                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += (float)part[t % (BEHIND + 1)][r] * f[pa][(pb * 16) / 128];
                             }
                             __builtin_amdgcn_sched_barrier(0);
                         }
@@ -1216,12 +1220,12 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 fa[a][0] = frag_a(stage, a, 0);
                 fa[a][1] = frag_a(stage, a, 1);
             }
-            v4f part[2];                                     // block scales: the partial products of two tiles
+            part_t part[2];                                  // block scales: the partial products of two tiles
             auto fold_tile = [&](int i) {
                 const int pa = i % C::TM, pb = i / C::TM;
                 const float f = as_cur[pa] * bs_cur[(pb * 16) / 128];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[i & 1][r] * f;
+                for (int r = 0; r < 4; ++r) acc[pa][pb][r] += (float)part[i & 1][r] * f;
             };
             v4i fball[READS_FIRST ? C::TN : 1][2];
             if constexpr (READS_FIRST) {
@@ -1249,7 +1253,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         // formed first is one multiply per row and K block instead of four per MFMA), one MFMA behind:
                         // the four FMAs of a tile go behind the MFMA of the next tile and run under it
                         const int i = b * C::TM + a;
-                        part[i & 1] = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], v4f{0, 0, 0, 0});
+                        part[i & 1] = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], part_t{0, 0, 0, 0});
                         if (i > 0) fold_tile(i - 1);
                     } else {
                         acc[a][b] = mma128<C::ARITH>(fb0, fb1, fa[a][0], fa[a][1], acc[a][b]);
@@ -1426,7 +1430,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             if (n >= p.N) continue;
             const size_t idx = (size_t)m * p.ldc + n;
             const bool full = p.vec_store && n + 3 < p.N;
-            if constexpr (C::ARITH == AR_I8) {
+            if constexpr (C::ARITH == AR_I8 && !C::BLOCK_SCALE) {
                 if (p.out_dtype == QGEMM_DT_I32) {
                     int *dst = (int *)Cz + idx;
                     if (full) *(v4i *)dst = acc[a][b];

@@ -35,7 +35,7 @@ struct SkinnyCfg {
     // an MFMA tile picked out of that with ds_bpermute); the scales of a round are requested in front of the round's
     // copies, so they have arrived wherever the copies they precede have.
     static constexpr bool BLOCK_SCALE = BLOCK_SCALE_;
-    static_assert(!BLOCK_SCALE_ || ARITH_ == AR_F8, "block scales are defined for fp8 only");
+    static_assert(!BLOCK_SCALE_ || ARITH_ == AR_F8 || ARITH_ == AR_I8, "block scales: fp8 and int8 operands");
     // TN = 4 (with TM = 4: a 64 x 64 tile): half the strips, so A is fetched half as often; for shapes with several
     // row tiles, where a CU's load path, not the stream of B from HBM, is what bounds a 32-column strip.
     static constexpr int TM = TM_, TN = TN_;                // 16 x 16 MFMA tiles of the workgroup's tile
@@ -62,7 +62,8 @@ template <class C>
 __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     extern __shared__ __attribute__((aligned(1024))) char smem[];
-    typedef typename AccT<C::ARITH>::type acc_t;
+    typedef typename AccT<C::ARITH>::type part_t;                       // one MFMA step: int32 for int8 operands, else fp32
+    typedef std::conditional_t<C::BLOCK_SCALE, v4f, part_t> acc_t;      // the running sums: fp32 with block scales
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     QGEMM_STAMP_DECL(6);
@@ -211,17 +212,17 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
                                                                                 as_cur[s][(16 * a) / 64])) * bs_cur[s];
             // one MFMA behind: the four FMAs of a tile go behind the MFMA of the next tile and run under it (straight
             // after their own MFMA they would wait for it, and the next MFMA for them)
-            v4f part[2];
+            part_t part[2];
 #pragma unroll
             for (int i = 0; i <= C::TM * C::TN; ++i) {
                 if (i < C::TM * C::TN) {
                     const int a = i % C::TM, b = i / C::TM;
-                    part[i & 1] = mma128<C::ARITH>(fb[s][b][0], fb[s][b][1], fa[s][a][0], fa[s][a][1], v4f{0, 0, 0, 0});
+                    part[i & 1] = mma128<C::ARITH>(fb[s][b][0], fb[s][b][1], fa[s][a][0], fa[s][a][1], part_t{0, 0, 0, 0});
                 }
                 if (i > 0) {
                     const int pa = (i - 1) % C::TM, pb = (i - 1) / C::TM;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[pa][pb][r] += part[(i - 1) & 1][r] * f[pa];
+                    for (int r = 0; r < 4; ++r) acc[pa][pb][r] += (float)part[(i - 1) & 1][r] * f[pa];
                 }
             }
         } else {
@@ -372,7 +373,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
         if (m >= p.M || n >= p.N) continue;
         const size_t idx = (size_t)m * p.ldc + n;
         const bool full = p.vec_store && n + 3 < p.N;
-        if constexpr (C::ARITH == AR_I8) {
+        if constexpr (C::ARITH == AR_I8 && !C::BLOCK_SCALE) {
             if (p.out_dtype == QGEMM_DT_I32) {
                 int *dst = (int *)Cz + idx;
                 if (full) *(v4i *)dst = s;

@@ -187,7 +187,7 @@ const Variant *table_for(int arith, bool block, int kmaj, int *count) {
     if (kmaj == 3) return (block && arith == AR_F8) ? variants_f8_block_tn(count) : nullptr;
     if (kmaj == 2) return block ? nullptr : (arith == AR_BF16 ? variants_bf16_nn(count) : (arith == AR_F16 ? variants_f16_nn(count) : nullptr));
     if (kmaj != 0) return nullptr;
-    if (block) return arith == AR_F8 ? variants_f8_block(count) : nullptr;
+    if (block) return arith == AR_F8 ? variants_f8_block(count) : (arith == AR_I8 ? variants_i8_block(count) : nullptr);
     switch (arith) {
         case AR_I8: return variants_i8(count);
         case AR_F8: return variants_f8(count);
@@ -671,7 +671,7 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
 #if QGEMM_DEBUG_BUILD
     a.dbg_cycles = (unsigned long long *)g_ctx.dbg_ptr;
 #endif
-    const bool i32_acc = q.arith == AR_I8;
+    const bool i32_acc = q.arith == AR_I8 && !q.block;        // (int8 with block scales sums in fp32)
     if (a.nsplit == 1) {
         a.C = (char *)q.C;
         a.ldc = (uint32_t)q.ldc;
@@ -1035,7 +1035,7 @@ QGEMM_EXPORT int qgemm_plan(int in_dtype, int scale_mode, int k_major, size_t M,
     if (arith < 0) return QGEMM_ERR_UNSUPPORTED;
     if (scale_mode != 0 && scale_mode != QGEMM_SCALE_PER_MATRIX && scale_mode != QGEMM_SCALE_BLOCK128)
         return QGEMM_ERR_INVALID_ARG;
-    if (scale_mode == QGEMM_SCALE_BLOCK128 && arith != AR_F8) return QGEMM_ERR_UNSUPPORTED;
+    if (scale_mode == QGEMM_SCALE_BLOCK128 && arith != AR_F8 && arith != AR_I8) return QGEMM_ERR_UNSUPPORTED;
     std::lock_guard<std::mutex> lock(g_ctx.mu);          // no device call below: 256 CUs are assumed before qgemm_init
     const size_t eb = (arith == AR_BF16 || arith == AR_F16) ? 2 : 1;
     NtProblem q;
@@ -1089,7 +1089,6 @@ QGEMM_EXPORT int qgemm_quantize(int in_dtype, int out_dtype, int mode, const voi
     if (out_dtype != QGEMM_DT_I8 && out_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
     if (mode != QGEMM_QUANT_PER_MATRIX && mode != QGEMM_QUANT_BLOCK_1x128 && mode != QGEMM_QUANT_BLOCK_128x128)
         return QGEMM_ERR_INVALID_ARG;
-    if (mode != QGEMM_QUANT_PER_MATRIX && out_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
     if (!scales) return QGEMM_ERR_INVALID_ARG;
     if (rows >= ((size_t)1 << 31) || cols >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
     std::lock_guard<std::mutex> lock(g_ctx.mu);
@@ -1231,7 +1230,8 @@ int scaled_gemm_entry(bool use_static, int in_dtype, int out_dtype, int scale_mo
     if (in_dtype != QGEMM_DT_I8 && in_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
     if (!out_dtype_ok(in_dtype, out_dtype)) return QGEMM_ERR_UNSUPPORTED;
     if (scale_mode != QGEMM_SCALE_PER_MATRIX && scale_mode != QGEMM_SCALE_BLOCK128) return QGEMM_ERR_INVALID_ARG;
-    if (scale_mode == QGEMM_SCALE_BLOCK128 && in_dtype != QGEMM_DT_F8E4M3) return QGEMM_ERR_UNSUPPORTED;
+    // (int8 with block scales and int32 output: there is no int32 sum of scaled blocks)
+    if (scale_mode == QGEMM_SCALE_BLOCK128 && out_dtype == QGEMM_DT_I32) return QGEMM_ERR_UNSUPPORTED;
     if (layout != QGEMM_LAYOUT_K_CONTIGUOUS && layout != QGEMM_LAYOUT_REFERENCE) return QGEMM_ERR_INVALID_ARG;
     if (split_k < 0) return QGEMM_ERR_INVALID_ARG;
     if (layout == QGEMM_LAYOUT_REFERENCE) {

@@ -32,6 +32,7 @@ struct Variant {
 const Variant *variants_i8(int *count);
 const Variant *variants_f8(int *count);
 const Variant *variants_f8_block(int *count);
+const Variant *variants_i8_block(int *count);
 const Variant *variants_bf16(int *count);
 const Variant *variants_f16(int *count);
 // K-major operand storage (GemmCfg::KMAJ): the reference's fp8 layout (A is K x M, B is K x N) and "NN" 16-bit GEMMs

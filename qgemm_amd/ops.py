@@ -2,6 +2,7 @@
 
   fp8_mm(a, b, as, bs, c)      src/mix_gemm/hip_mix_gemm_kernel.cpp:508-516
   int8_mm / bf16_mm            the stubs in src/gemm/sm80_gemm_kernel.cu:4-22
+  int8_mm_block                int8 operands with the 128-block scales of fp8_mm (no counterpart in the reference)
   matrix_transpose(in, out)    src/transpose/transpose.cu:60-74
   gemm(...)                    GEMM_kernel_v*<In, Out> of include/gemm.h:25-66
   quantize(x, ...)             the Q_A / Q_B of README.md:1 (the reference has no quantiser)
@@ -157,6 +158,19 @@ def int8_mm(a, b, a_scale, b_scale, c, split_k=0):
     _need_out(c, m, n)
     return scaled_gemm(a, b, a_scale, b_scale, c, m, n, k, SCALE_PER_MATRIX, split_k=split_k, in_dtype=DT_I8,
                        ldC=c.stride(0))
+
+
+def int8_mm_block(a, b, a_scale, b_scale, c, split_k=0):
+    """int8 GEMM with 128-block scales, the int8 twin of fp8_mm's arithmetic (hip_mix_gemm_kernel.cpp:231-244) on
+    K-contiguous operands: a [m,k] int8, b [n,k] int8, a_scale [m, ceil(k/128)] and b_scale [ceil(n/128), ceil(k/128)]
+    fp32 row-major, c [m,n] fp32 / bf16 / fp16.  Every 128-wide K block's exact int32 partial is folded into an fp32
+    sum with a_scale[m, kb] * b_scale[n // 128, kb]."""
+    m, k = a.shape
+    n = b.shape[0]
+    if a.dtype != torch.int8 or b.dtype != torch.int8:
+        raise TypeError(f"int8_mm_block takes int8 operands, got {a.dtype} and {b.dtype}")
+    _need_out(c, m, n)
+    return scaled_gemm(a, b, a_scale, b_scale, c, m, n, k, SCALE_BLOCK128, split_k=split_k, in_dtype=DT_I8, ldC=c.stride(0))
 
 
 def bf16_mm(a, b, c):

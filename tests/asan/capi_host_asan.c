@@ -53,7 +53,7 @@ int main(void) {
     {
         const int nb = qgemm_variant_count(QGEMM_DT_F8E4M3, QGEMM_SCALE_BLOCK128, 0);
         const int ni = qgemm_variant_count(QGEMM_DT_I8, QGEMM_SCALE_PER_MATRIX, 0);
-        CHECK(nb > 4 && ni > 4 && qgemm_variant_count(99, 1, 0) == 0 && qgemm_variant_count(QGEMM_DT_I8, QGEMM_SCALE_BLOCK128, 0) == 0);
+        CHECK(nb > 4 && ni > 4 && qgemm_variant_count(99, 1, 0) == 0 && qgemm_variant_count(QGEMM_DT_BF16, QGEMM_SCALE_BLOCK128, 0) == 0);
         CHECK(qgemm_variant_name(QGEMM_DT_I8, 1, 0, ni, buf, sizeof buf) == QGEMM_ERR_INVALID_ARG);
         CHECK(qgemm_variant_name(QGEMM_DT_I8, 1, 0, 0, NULL, 0) == QGEMM_ERR_INVALID_ARG);
         for (int v = 0; v < nb + ni; ++v) {
@@ -104,11 +104,11 @@ int main(void) {
     CHECK(qgemm_gemm(QGEMM_DT_BF16, QGEMM_DT_F32, 1, p, 16, p, 16, p, 16, 0, 16, 16, NULL) == QGEMM_OK);
     CHECK(qgemm_scaled_gemm(QGEMM_DT_F8E4M3, QGEMM_DT_BF16, 2, 1, p, p, NULL, NULL, p, 64, 48, 64, 128, 0, NULL) == QGEMM_ERR_NOT_DIVISIBLE_M);
     CHECK(qgemm_scaled_gemm(QGEMM_DT_F8E4M3, QGEMM_DT_BF16, 2, 0, p, p, NULL, NULL, p, 64, 64, 64, 128, 0, NULL) == QGEMM_ERR_INVALID_ARG);
-    CHECK(qgemm_scaled_gemm_static(QGEMM_DT_I8, QGEMM_DT_F32, 2, 0, p, p, p, p, p, 64, 64, 64, 128, 0, NULL) == QGEMM_ERR_UNSUPPORTED);
+    CHECK(qgemm_scaled_gemm_static(QGEMM_DT_I8, QGEMM_DT_I32, 2, 0, p, p, p, p, p, 64, 64, 64, 128, 0, NULL) == QGEMM_ERR_UNSUPPORTED);
     CHECK(qgemm_transpose(3, p, p, 4, 4, NULL) == QGEMM_ERR_UNSUPPORTED);
     CHECK(qgemm_transpose(2, p, p, (size_t)1 << 31, 4, NULL) == QGEMM_ERR_TOO_LARGE);
     CHECK(qgemm_quantize(QGEMM_DT_I8, QGEMM_DT_I8, 1, p, 4, 4, 4, p, 4, (float *)p, 0, 0, NULL) == QGEMM_ERR_UNSUPPORTED);
-    CHECK(qgemm_quantize(QGEMM_DT_F32, QGEMM_DT_I8, 2, p, 4, 4, 4, p, 4, (float *)p, 0, 0, NULL) == QGEMM_ERR_UNSUPPORTED);
+    CHECK(qgemm_quantize(QGEMM_DT_F32, QGEMM_DT_F32, 2, p, 4, 4, 4, p, 4, (float *)p, 0, 0, NULL) == QGEMM_ERR_UNSUPPORTED);
     void *base = p;
     size_t bytes = 7;
     CHECK(qgemm_workspace_info(&base, &bytes) == QGEMM_OK && qgemm_workspace_info(NULL, NULL) == QGEMM_ERR_INVALID_ARG);

@@ -48,9 +48,9 @@ def test_argument_validation_needs_no_device():
     assert lib.qgemm_gemm(Q.DT_BF16, Q.DT_I32, 1, one, 16, one, 16, one, 16, 16, 16, 16, None) == 2
     # bad layout enum, leading dimension smaller than the row
     assert lib.qgemm_gemm(Q.DT_BF16, Q.DT_F32, 7, one, 16, one, 16, one, 16, 16, 16, 16, None) == 1
-    # scaled: only int8 / fp8 inputs; block scales only for fp8; reference layout checks divisibility first
+    # scaled: only int8 / fp8 inputs; no int32 output with block scales; reference layout checks divisibility first
     assert lib.qgemm_scaled_gemm(Q.DT_BF16, Q.DT_F32, 1, 0, one, one, one, one, one, 16, 16, 16, 16, 0, None) == 2
-    assert lib.qgemm_scaled_gemm(Q.DT_I8, Q.DT_F32, 2, 0, one, one, one, one, one, 16, 16, 16, 16, 0, None) == 2
+    assert lib.qgemm_scaled_gemm(Q.DT_I8, Q.DT_I32, 2, 0, one, one, one, one, one, 16, 16, 16, 16, 0, None) == 2
     assert lib.qgemm_scaled_gemm(Q.DT_F8E4M3, Q.DT_BF16, 2, 1, one, one, one, one, one, 64, 48, 64, 128, 0, None) == 6
     assert lib.qgemm_scaled_gemm(Q.DT_F8E4M3, Q.DT_BF16, 2, 1, one, one, one, one, one, 48, 64, 48, 128, 0, None) == 7
     assert lib.qgemm_scaled_gemm(Q.DT_F8E4M3, Q.DT_BF16, 2, 1, one, one, one, one, one, 64, 64, 64, 80, 0, None) == 8
@@ -188,7 +188,7 @@ def test_plan_names_the_kernel_without_a_device():
         Q.force_config(None)
         Q.set_option("force_split", 0)
     with pytest.raises(Q.QgemmError):
-        plan(Q.DT_I8, Q.SCALE_BLOCK128, 0, 256, 256, 256)        # block scales are fp8 only
+        plan(Q.DT_BF16, Q.SCALE_BLOCK128, 0, 256, 256, 256)      # block scales: fp8 and int8 operands
     with pytest.raises(Q.QgemmError):
         plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 0, 256, 256)
 

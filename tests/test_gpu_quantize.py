@@ -90,8 +90,8 @@ def test_16_bit_inputs_and_row_stride(dt):
 def test_errors_and_empty():
     say("quantize errors")
     x = torch.zeros((16, 128), device="cuda")
-    with pytest.raises(Q.QgemmError) as e:                   # block scales are defined for fp8 only
-        Q.quantize(x, torch.int8, Q.QUANT_BLOCK_1x128)
+    with pytest.raises(Q.QgemmError) as e:                   # the output is int8 or e4m3
+        Q.quantize(x, torch.int32, Q.QUANT_BLOCK_1x128)
     assert e.value.status == 2
     q, s = Q.quantize(x, torch.float8_e4m3fn, Q.QUANT_PER_MATRIX)      # all zeros: s = 1
     assert host(s)[0] == 1.0 and not _u8(q).any()

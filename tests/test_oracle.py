@@ -327,6 +327,41 @@ def test_block_scaled_reference_layouts_agree():
     assert np.array_equal(nt, tn)
 
 
+def test_int8_block_scaled_pinned_without_itself():
+    """ref_gemm_i8_block (int8 operands, 128-block scales): brute force in Python integers and numpy float32 steps on a
+    lattice of entries (a dropped block, a scale taken from the wrong row / K block / column block, or a partial
+    converted too late shows); unit scales give the exact int32 GEMM; power-of-two scales commute exactly; equal scales
+    are the per-matrix product up to one rounding per block; a partial last K block; both storages agree."""
+    M, N, K = 24, 256, 400                              # K: three whole blocks and one of 16
+    KB = (K + 127) // 128
+    qa = R.quantize_int8(R.fill_normal((M, K), 61))[0]
+    qb = R.quantize_int8(R.fill_normal((N, K), 62))[0]
+    as_ = R.fill_uniform((M, KB), 63, 0.5, 2.0)
+    bs = R.fill_uniform((N // 128, KB), 64, 0.5, 2.0)
+    got = R.gemm_i8_block(qa, qb, as_, bs)
+    for m in range(0, M, 5):
+        for n in range(0, N, 37):
+            acc = np.float32(0)
+            for kb in range(KB):
+                p = sum(int(qa[m, k]) * int(qb[n, k]) for k in range(kb * 128, min(K, kb * 128 + 128)))   # exact
+                acc = np.float32(acc + np.float32(np.float32(np.float32(p) * as_[m, kb]) * bs[n // 128, kb]))
+            assert got[m, n] == acc, (m, n)
+    exact = R.gemm_i8_i32(qa, qb)
+    ones_a, ones_b = np.ones((M, KB), np.float32), np.ones((N // 128, KB), np.float32)
+    assert np.array_equal(R.gemm_i8_block(qa, qb, ones_a, ones_b), exact.astype(np.float32))     # |acc| < 2^24 here
+    assert np.abs(exact).max() < 2 ** 24
+    assert np.array_equal(R.gemm_i8_block(qa, qb, ones_a * 8, ones_b * 0.25), exact.astype(np.float32) * 2)
+    sa, sb = np.float32(1.37), np.float32(0.61)
+    pm = R.gemm_i8_block(qa, qb, ones_a * sa, ones_b * sb).astype(np.float64)
+    assert np.allclose(pm, exact.astype(np.float64) * float(sa) * float(sb), rtol=1e-6, atol=1e-2)
+    assert not np.allclose(got, R.gemm_i8_block(qa, qb, as_[::-1].copy(), bs), rtol=1e-3)
+    assert not np.allclose(got, R.gemm_i8_block(qa, qb, as_, bs[::-1].copy()), rtol=1e-3)
+    assert not np.allclose(got, R.gemm_i8_block(qa, qb, as_[:, ::-1].copy(), bs), rtol=1e-3)
+    tn = R.gemm_i8_block(np.ascontiguousarray(qa.T), np.ascontiguousarray(qb.T), np.ascontiguousarray(as_.T),
+                         np.ascontiguousarray(bs.T), "tn", "col")
+    assert np.array_equal(got, tn)
+
+
 def test_reference_tile_dispatch_and_swizzle():
     # hip_mix_gemm_kernel.cpp:442-505
     assert [R.select_tile(d, "m") for d in (6144, 192, 96, 48)] == [128, 64, 32, 0]
