@@ -364,7 +364,10 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     // or with 64 tiles and 64 K steps; beyond 64 K steps the tiles with a K split across workgroups catch up
     // (bf16 256 x 2048 x 7168, 112 steps: 18.9 against 22.9 us).  With block scales the gain is larger, the small tiles
     // of the simple pipeline being slower there: 512 x 2048 x 4096 18.3 -> 11.7 us, 256 x 4096 x 4096 17.8 -> 11.8.
-    if (vi >= 0 && !kmaj && M > 128 && ksteps >= 16 && ksteps <= 64) {
+    // From 65 rows on: with two row tiles a workgroup pulls half of A (an L2 hit, but through its CU's load path) next
+    // to twice the strip of B, 256 KiB instead of 320 KiB at 128 x 7168 x 2048, the smallest sum a tile of that area
+    // has (config 5 at M = 128, B out of HBM: 8.9 -> 8.3 us; M = 64 stays on 32-column strips, 6.8 us).
+    if (vi >= 0 && !kmaj && M > 64 && ksteps >= 16 && ksteps <= 64) {
         const size_t t64 = ((M + 63) / 64) * ((N + 63) / 64);
         if (t64 <= (size_t)cus && (t64 >= 128 || (t64 >= 64 && ksteps <= 32)))
             for (int i = 0; i < count; ++i)

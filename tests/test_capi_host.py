@@ -109,7 +109,7 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8_ks"
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168 - 128) == "256x256_w2x4_solo8"
     # config 5: the skinny-M kernel (K split over the eight waves of a workgroup)
-    for m, name in ((16, "skinny_16x32_k8"), (64, "skinny_64x32_k8"), (128, "skinny_128x32_k8")):
+    for m, name in ((16, "skinny_16x32_k8"), (64, "skinny_64x32_k8"), (128, "skinny_64x64_k8")):
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
         assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 24, 4096, 4096) == "skinny_32x32_k8"
@@ -122,8 +122,8 @@ def test_plan_names_the_kernel_without_a_device():
     # fit one round and K is not long: the skinny-M kernel rather than what the estimate (of resident operands) likes
     assert plan(Q.DT_BF16, 0, 0, 64, 14336, 4096) == "skinny_64x64_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 8192, 8192) == "skinny_64x32_k8"
-    assert plan(Q.DT_BF16, 0, 0, 128, 7168, 2048) == "skinny_128x32_k8"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 8192, 8192) == "skinny_128x32_k8"
+    assert plan(Q.DT_BF16, 0, 0, 128, 7168, 2048) == "skinny_64x64_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 8192, 8192) == "skinny_64x64_k8"
     assert plan(Q.DT_BF16, 0, 0, 128, 8192, 8192) == "128x128_w2x2_k2_splitk4"
     # ... but not with few K steps or where the estimate prefers wide tiles
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 7168, 512) == "128x32_w4x1_dma"
@@ -153,8 +153,8 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 6144, 6144) == "256x256_w2x4_solo8_ks+256x128_w2x2_cw_ks"
     # ... also when a single launch would take smaller tiles for everything, and with a rest of at most 128 rows
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 5000, 4096, 7168) == "256x256_w2x2_solo+128x128_w2x2_k2"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 7000, 7168, 2048) == "256x256_w2x2_solo+skinny_128x32_k8"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 7000, 7168, 2048) == "256x256_w2x4_solo8_ks+skinny_128x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 7000, 7168, 2048) == "256x256_w2x2_solo+skinny_64x64_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 7000, 7168, 2048) == "256x256_w2x4_solo8_ks+skinny_64x64_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 4096, 14336, 4096) == "256x256_w2x2_solo"     # 3.5 rounds: no gain
     Q.set_option("row_split", 0)
     try:

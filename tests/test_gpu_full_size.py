@@ -289,7 +289,7 @@ def test_row_split_of_a_partly_empty_last_round():
     assert_close(host(c16)[rows], R.gemm_f32acc(R.decode_bf16(ha[rows]), R.decode_bf16(hb)), rtol=1e-4, atol=1e-3, what=name)
 
 
-@pytest.mark.parametrize("shape,m_main,rest", [((4184, 4096, 2048), 4096, "skinny_128x32_k8"),     # 88 rows below one full round
+@pytest.mark.parametrize("shape,m_main,rest", [((4184, 4096, 2048), 4096, "skinny_64x64_k8"),      # 88 rows below one full round
                                                ((5000, 4096, 2048), 4096, "128x128")])            # single launch: 128 x 128 tiles
 def test_row_split_with_a_short_rest_and_against_smaller_tiles(shape, m_main, rest):
     """Row split where the rows below the full rounds are at most 128 (they go to the skinny-M kernel) and where a
