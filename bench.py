@@ -592,7 +592,14 @@ def main():
         bs4t = torch.rand(n4 // 128, kb4t, device=dev) * 1.5 + 0.5
         extra["cfg4_shape_k7200_partial_last_k_block"] = gemm_entry(
             tx(lambda: Q.scaled_gemm(a4t, b4t, as4t, bs4t, c4, m4, n4, k4t, Q.SCALE_BLOCK128)), 2.0 * m4 * n4 * k4t, PEAK_TFLOPS["f8"])
-        del a4t, b4t, c4
+        del a4t, b4t
+        # int8 operands with the same 128-block scales (each K block's exact int32 partial folded into an fp32 sum): the
+        # int8 twin of the reference's block-scaled arithmetic, config 4's shape
+        a4i, _ = _quant_i8(torch.randn(m4, k4, device=dev))
+        b4i, _ = _quant_i8(torch.randn(n4, k4, device=dev))
+        extra["cfg4_shape_int8_block_scales"] = gemm_entry(
+            tx(lambda: Q.int8_mm_block(a4i, b4i, as4, bs4, c4)), f4, PEAK_TFLOPS["i8"])
+        del a4i, b4i, c4
         # cfg 5: skinny M, N = 7168, K = 2048, int8 (f32 out) and fp8 (bf16 out); bandwidth-bound: GB/s of algorithmic
         # bytes.  "rotated": every launch of the graph reads another B (24 buffers, 352 MB: more than the Infinity
         # Cache holds); "resident": all 24 launches read the same B.
