@@ -1,5 +1,5 @@
 """Seeded random sweep over what the dispatch can combine: family (int8 / fp8 per matrix / fp8 block scales in both
-storages / bf16 / fp16 with B stored N x K or K x N), shape (ragged, down to one row), tile variant (the
+storages / int8 block scales / bf16 / fp16 with B stored N x K or K x N), shape (ragged, down to one row), tile variant (the
 heuristic's or a forced row of the table), K split and output type.  Every case is checked against the CPU oracle:
 int32 accumulators bit for bit, float outputs to rtol 2e-2 / atol 1e-2 (plus half an ulp of a 16-bit output)."""
 import numpy as np
@@ -15,6 +15,7 @@ pytestmark = pytest.mark.gpu
 ROWS = {
     "i8": Q.variant_names(Q.DT_I8, Q.SCALE_PER_MATRIX), "f8": Q.variant_names(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX),
     "f8_block": Q.variant_names(Q.DT_F8E4M3, Q.SCALE_BLOCK128), "f8_block_ref": Q.variant_names(Q.DT_F8E4M3, Q.SCALE_BLOCK128),
+    "i8_block": Q.variant_names(Q.DT_I8, Q.SCALE_BLOCK128),
     "bf16_nk": Q.variant_names(Q.DT_BF16), "bf16_kn": Q.variant_names(Q.DT_BF16),
     "f16_nk": Q.variant_names(Q.DT_F16), "f16_kn": Q.variant_names(Q.DT_F16),
 }
@@ -28,8 +29,8 @@ def _reset_options():
 
 
 def _draw(rng):
-    fam = rng.choice(["i8", "f8", "f8_block", "f8_block_ref", "bf16_nk", "bf16_kn", "f16_nk", "f16_kn"])
-    kq = {"i8": 128, "f8": 128, "f8_block": 128, "f8_block_ref": 128}.get(fam, 64)     # elements of a 128-byte K step
+    fam = rng.choice(["i8", "f8", "f8_block", "f8_block_ref", "i8_block", "bf16_nk", "bf16_kn", "f16_nk", "f16_kn"])
+    kq = {"i8": 128, "f8": 128, "f8_block": 128, "f8_block_ref": 128, "i8_block": 128}.get(fam, 64)     # elements of a 128-byte K step
     K = int(rng.integers(1, 9)) * kq
     if rng.random() < 0.25:                         # a long K: several rounds of the skinny-M kernel, deep rings
         K = int(rng.integers(9, 41)) * kq
@@ -48,12 +49,12 @@ def _draw(rng):
     # (a K-major call whose family lacks the forced row goes through the transposes to the K-contiguous row of that name)
     variant = str(rng.choice(ROWS[fam])) if rng.random() < 0.6 else None
     split = int(rng.choice([0, 0, 0, 2, 3])) if K // kq >= 4 else 0
-    if fam.startswith("f8_block") and split and (K + 127) // 128 < 2 * split:
+    if "block" in fam and split and (K + 127) // 128 < 2 * split:
         split = 0
     return fam, M, N, K, variant, split
 
 
-@pytest.mark.parametrize("seed", range(128))
+@pytest.mark.parametrize("seed", range(192))
 def test_random_case(seed):
     rng = np.random.default_rng(1000 + seed)
     fam, M, N, K, variant, split = _draw(rng)
@@ -79,6 +80,13 @@ def test_random_case(seed):
         qb, sb = R.quantize_fp8(R.fill_normal((N, K), seed + 500))
         ref = R.gemm_f32acc(R.decode_fp8(qa), R.decode_fp8(qb)) * np.float32(sa * sb)
         Q.scaled_gemm(fp8_tensor(qa), fp8_tensor(qb), scalar(sa), scalar(sb), c, M, N, K, Q.SCALE_PER_MATRIX)
+    elif fam == "i8_block":
+        qa, _ = R.quantize_int8(R.fill_normal((M, K), seed))
+        qb, _ = R.quantize_int8(R.fill_normal((N, K), seed + 500))
+        as_ = R.fill_uniform((M, (K + 127) // 128), seed + 1, 0.5, 2.0) / np.float32(127)
+        bs = R.fill_uniform(((N + 127) // 128, (K + 127) // 128), seed + 2, 0.5, 2.0) / np.float32(127)
+        ref = R.gemm_i8_block(qa, qb, as_, bs)
+        Q.int8_mm_block(dev(qa), dev(qb), dev(as_), dev(bs), c)
     elif fam in ("f8_block", "f8_block_ref"):
         qa, _ = R.quantize_fp8(R.fill_normal((M, K), seed))
         qb, _ = R.quantize_fp8(R.fill_normal((N, K), seed + 500))
