@@ -187,6 +187,16 @@ def test_plan_names_the_kernel_without_a_device():
     finally:
         Q.force_config(None)
         Q.set_option("force_split", 0)
+    # a name no family has is refused when it is set; a name the problem's family lacks when a problem asks for it
+    with pytest.raises(Q.QgemmError):
+        Q.force_config("no_such_row")
+    Q.force_config("256x256_w2x2_solo")                          # (not among the block-scaled rows)
+    try:
+        with pytest.raises(Q.QgemmError):
+            plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168)
+        assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 4608, 7168) == "256x256_w2x2_solo"
+    finally:
+        Q.force_config(None)
     with pytest.raises(Q.QgemmError):
         plan(Q.DT_BF16, Q.SCALE_BLOCK128, 0, 256, 256, 256)      # block scales: fp8 and int8 operands
     with pytest.raises(Q.QgemmError):
