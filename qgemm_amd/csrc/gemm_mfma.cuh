@@ -105,7 +105,7 @@ struct GemmCfg {
     // ones 64 requests, which these tiles (a step of several hundred cycles per wave) can afford and which saves the
     // launch that would copy the scales into the other order.
     static constexpr bool AS_ANY_STRIDE = BLOCK_SCALE_ && PIPE_ != PIPE_SOLO;
-    // STAGES (simple pipeline, DMA loader): number of LDS stages, 0 = chosen below.
+    // STAGES (simple pipeline): number of LDS stages, 0 = chosen below.
     // KGROUPS = 2: the workgroup has two sets of WAVES_M x WAVES_N waves and two waves that copy; set 0 computes
     // the even K steps and set 1 the odd ones of the same tile, half a turn apart, and the two partial sums meet in
     // LDS before the epilogue.  A tile that is alone on its CU (a shape with no more tiles than CUs) otherwise
@@ -137,7 +137,7 @@ struct GemmCfg {
     static constexpr int A_BYTES = RBA * 2048, B_BYTES = RBB * 2048;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int LPT_A = RBA * 2 / NW;                  // A load instructions per wave
-    // simple pipeline with the DMA loader: as many stages in flight as LDS and the 6-bit vmcnt allow (at most
+    // simple pipeline: as many stages in flight as LDS and the 6-bit vmcnt allow (at most
     // 8).  A workgroup that streams a narrow strip of B (skinny M) otherwise waits one full memory round trip
     // per K step.  The block-scale form keeps two (its scale loads share vmcnt with the copies), except with K
     // groups, where the scales travel to LDS like the operands.

@@ -761,7 +761,7 @@ bool settle_scale_layout(const NtProblem &q, Plan &pl) {
         return true;
     }
     // some other arrangement (K-contiguous, as QGEMM_LAYOUT_K_CONTIGUOUS passes it): fine where every launch of the
-    // plan either takes any strides (simple and ping-pong pipelines) or has a twin for it
+    // plan either takes any strides (simple pipeline, skinny-M kernel) or has a twin for it
     // (a twin fetches the scales of Variant::ks_blocks K blocks of a row per load, two or four: rows aligned to that
     // many floats, K and every K slice a multiple of that many blocks)
     bool as_is = true;
@@ -1496,7 +1496,7 @@ QGEMM_EXPORT int qgemm_selftest_layouts(char *buf, size_t buflen) {
                                   z ? "IS" : "is NOT");
                     rep += line;
                     // tile rows past M or N are kept out of reach by the range check alone (the row block of a
-                    // copy sits in the scalar offset in the simple and ping-pong pipelines)
+                    // copy sits in the scalar offset in the simple pipeline)
                     if (!z) all_ok = false;
                     continue;
                 }
