@@ -618,7 +618,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // two K blocks of its row at once, on every other step, so the 64 rows of a load, 64 requests of their
             // own, cost the texture addresser half of what one strided dword per step would.  Either way block kb
             // sits in component kb & 1 of as_pair.
-            float as_b[TMs], bs_c[NBS], sc[2][NBS];
+            float as_b[TMs], bs_c[NBS], sc[2][NBS] = {};        // (sc: zero until the first row of the first step has set it)
             v2i as_pair[NLD];
             constexpr bool as_kcont = C::ASK;
             // Copying waves and K-contiguous a_scale (the twin `_ks` of the row with copying waves): the computing waves
@@ -714,8 +714,15 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // (generic_tag: the form of the step outside the unrolled groups.  Only there can the copies a step issues,
             // those of step kt + 2, be the ones of a partial last K step: they carry the OR that puts the lanes past
             // the end of K out of range, 0 for every other step.)
-            auto step = [&](int kt, int par, auto generic_tag) {             // par = kt & 1
+            // Block scales: the partial product of the last tile of a step is folded behind the first MFMA of the next
+            // step instead of at the end of its own, where the wave would wait out that MFMA with nothing else to
+            // issue (CARRY: the steps of the unrolled groups, all alike, so that they stay one instantiation; the
+            // first of them folds a zero, and what the last leaves over is folded behind the group loop).
+            constexpr int BEHIND = 2;          // MFMAs between a partial product and its fold
+            part_t left_over = {0, 0, 0, 0};   // the partial product a step leaves to the next
+            auto step = [&](int kt, int par, auto generic_tag, auto carry_tag) {             // par = kt & 1
                 constexpr bool GENERIC = decltype(generic_tag)::value;
+                constexpr bool CARRY = decltype(carry_tag)::value && C::BLOCK_SCALE;
                 const uint32_t tor = GENERIC ? (kt + 2 == kt_tail ? tail_or : 0u) : 0u;
                 const int a_nx = next_buf(a_rd);
                 constexpr bool copies = !C::COPYW;            // (the copying waves' loop is below)
@@ -725,7 +732,6 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 // copies: by the time they are used nothing older is in flight).  The factor of row a,
                 // a_scale[row] * b_scale, is made one row ahead: the cross-lane pick behind the first
                 // MFMA of row a-1, the multiply behind the second MFMA of row a, so two factors are live at a time.
-                constexpr int BEHIND = 2;      // MFMAs between a partial product and its fold
                 part_t part[BEHIND + 1];
                 fetch_a_scales(kt + 1, par ^ 1);
                 fetch_b_scales(kt + 1);
@@ -745,6 +751,15 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         const float f = sc[pa % 2][(pb * 16) / 128];
 #pragma unroll
                         for (int r = 0; r < 4; ++r) acc[pa][pb][r] += (float)part[i % (BEHIND + 1)][r] * f;
+                    }
+                };
+                // the last tile of the step before (its factor is still in sc: a row's factor is replaced behind the
+                // second MFMA of the same row of the next step at the earliest)
+                auto fold_left_over = [&]() {
+                    if constexpr (C::BLOCK_SCALE) {
+                        const float f = sc[(TMs - 1) % 2][((C::TN - 1) * 16) / 128];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[TMs - 1][C::TN - 1][r] += (float)left_over[r] * f;
                     }
                 };
                 // the side instructions of a row go between its MFMAs, one at a time: a run of them in front
@@ -827,6 +842,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                             }
                             __builtin_amdgcn_sched_barrier(0);
                             if (i >= BEHIND) fold(i - BEHIND);
+                            else if (CARRY && i == 0) fold_left_over();
                             __builtin_amdgcn_sched_barrier(0);
                         } else {
                             mma(a, b, 0);
@@ -839,7 +855,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                 }
                 if constexpr (C::BLOCK_SCALE) {
 #pragma unroll
-                    for (int i = TMs * C::TN - BEHIND; i < TMs * C::TN; ++i) fold(i);
+                    for (int i = TMs * C::TN - BEHIND; i < TMs * C::TN - (CARRY ? 1 : 0); ++i) fold(i);
+                    if constexpr (CARRY) left_over = part[(TMs * C::TN - 1) % (BEHIND + 1)];
                     rotate_scales(par ^ 1, kt + 1);
                 }
                 a_rd = a_nx;
@@ -939,17 +956,22 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         for (int j = 0; j < 6; ++j) {
                             a_rd = j % 3;
                             a_wr = (j + 2) % 3;
-                            step(kt + j, j & 1, no_t{});
+                            step(kt + j, j & 1, no_t{}, yes_t{});
                         }
+                    }
+                    if constexpr (C::BLOCK_SCALE && !PINNED) {       // what the last step of the groups left over
+                        const float f = sc[(TMs - 1) % 2][((C::TN - 1) * 16) / 128];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[TMs - 1][C::TN - 1][r] += (float)left_over[r] * f;
                     }
                     a_rd = 0;            // kt is a multiple of six here
                     a_wr = 2;
                 }
                 for (; kt + 2 <= nk; kt += 2) {
-                    step(kt, 0, yes_t{});
-                    step(kt + 1, 1, yes_t{});
+                    step(kt, 0, yes_t{}, no_t{});
+                    step(kt + 1, 1, yes_t{}, no_t{});
                 }
-                if (kt < nk) step(kt, 0, yes_t{});
+                if (kt < nk) step(kt, 0, yes_t{}, no_t{});
                 __builtin_amdgcn_s_waitcnt(0x0070);      // copies landed, reads done, before LDS serves the epilogue
                 phase_barrier();
                 // the MFMAs above are opaque to the compiler's hazard handling: give the last one its wait states
