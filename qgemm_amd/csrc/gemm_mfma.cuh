@@ -613,9 +613,10 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
             // the other; v_permlane32_swap: upper half against lower half).  The same pick through ds_bpermute
             // shares the LDS queue, which answers in order, with the fragment reads issued two rows ahead: waiting
             // for a pick then means waiting for those reads as well (7 % of the K loop on config 4).
-            // a_scale as the caller has it, K blocks contiguous (GemmCfg::ASK; the host picks that kernel only with an
-            // even number of K blocks per row and per K slice and 8-byte aligned rows): lane l fetches the scales of
-            // two K blocks of its row at once, on every other step, so the 64 rows of a load, 64 requests of their
+            // a_scale as the caller has it, K blocks contiguous (GemmCfg::ASK): lane l fetches the scales of
+            // two K blocks of its row at once with an 8-byte load (4-byte alignment is enough; behind a row's last
+            // block the second half is the next row's first scale or, past the end of the array, the zero of the
+            // range check: nobody uses it), on every other step, so the 64 rows of a load, 64 requests of their
             // own, cost the texture addresser half of what one strided dword per step would.  Either way block kb
             // sits in component kb & 1 of as_pair.
             float as_b[TMs], bs_c[NBS], sc[2][NBS] = {};        // (sc: zero until the first row of the first step has set it)

@@ -745,7 +745,7 @@ int launch_transpose(int elem_bytes, const void *in, void *out, size_t M, size_t
 // Which arrangement of a_scale the kernels of a block-scaled plan read.  Most want it rows-contiguous
 // (a_scale[m + kb * ld], what QGEMM_LAYOUT_REFERENCE passes); the block-scaled 8-wave solo kernel has a twin
 // (GemmCfg::ASK, table name "<name>_ks") that reads it with the K blocks contiguous, as QGEMM_LAYOUT_K_CONTIGUOUS
-// passes it, two K blocks per load: rows 8-byte aligned, an even number of K blocks per row and per K slice.
+// passes it, two K blocks per 8-byte load (any number of K blocks per row and per K slice: see below).
 // Puts the right one of each pair into the plan.  Returns true when the plan then reads q's scales as they are,
 // false when they first have to be copied rows-contiguous (scales_rows_contiguous).
 bool settle_scale_layout(const NtProblem &q, Plan &pl) {
@@ -774,8 +774,13 @@ bool settle_scale_layout(const NtProblem &q, Plan &pl) {
             break;
         }
         const uint32_t g = (uint32_t)twin->ks_blocks;
-        as_is = g > 0 && q.as_ms % g == 0 && ((uintptr_t)q.as % (4 * g)) == 0 && p->a.ksteps % g == 0 &&
-                !(p->a.nsplit > 1 && p->a.ksteps_per_split % g != 0);
+        // (two K blocks per load, into registers: any row length and any slice.  An 8-byte buffer load needs 4-byte
+        // alignment only, the pair that starts with a row's last block ends with the next row's first, which nobody
+        // uses, and at the end of the array the range check, which is per dword, returns zero for it: probed by
+        // qgemm_selftest_layouts.  Four blocks per copy go through LDS and keep their alignment rules.)
+        as_is = g == 2 ? ((uintptr_t)q.as % 4) == 0
+                       : (g > 0 && q.as_ms % g == 0 && ((uintptr_t)q.as % (4 * g)) == 0 && p->a.ksteps % g == 0 &&
+                          !(p->a.nsplit > 1 && p->a.ksteps_per_split % g != 0));
     }
     for (Plan *p = &pl; p; p = p->rest.get()) {
         if (p->v->a_scale_any_stride) continue;
@@ -1521,6 +1526,33 @@ QGEMM_EXPORT int qgemm_selftest_layouts(char *buf, size_t buflen) {
         (void)hipFree(dsrc);
         (void)hipFree(doff);
         (void)hipFree(dout);
+    }
+
+    // ---- 8-byte buffer loads at 4-byte aligned offsets, and across the end of the buffer range: the twin kernels
+    //      for K-contiguous a_scale (two K blocks per load) read rows with an odd number of K blocks that way
+    {
+        const int n_in = 60;                                 // floats inside the range; 64 are allocated
+        std::vector<float> h(64);
+        for (int i = 0; i < 64; ++i) h[i] = 100.0f + (float)i;
+        void *d = nullptr, *o = nullptr;
+        HIP_TRY(hipMalloc(&d, 64 * 4));
+        HIP_TRY(hipMalloc(&o, 128 * 4));
+        HIP_TRY(hipMemcpy(d, h.data(), 64 * 4, hipMemcpyHostToDevice));
+        hipLaunchKernelGGL(probe_b64_load_kernel, dim3(1), dim3(64), 0, 0, (const float *)d, (uint32_t)(n_in * 4), (int *)o);
+        HIP_TRY(hipGetLastError());
+        std::vector<float> got(128);
+        HIP_TRY(hipMemcpy(got.data(), o, 128 * 4, hipMemcpyDeviceToHost));
+        int bad = 0;
+        for (int l = 0; l + 1 < n_in; ++l) bad += got[2 * l] != h[l] || got[2 * l + 1] != h[l + 1];
+        const bool per_dword = got[2 * (n_in - 1)] == h[n_in - 1] && got[2 * (n_in - 1) + 1] == 0.0f;
+        bool beyond_zero = true;
+        for (int l = n_in; l < 64; ++l) beyond_zero &= got[2 * l] == 0.0f && got[2 * l + 1] == 0.0f;
+        std::snprintf(line, sizeof(line), "b64 buffer load: mismatched_pairs=%d (odd lanes are 4-byte aligned only), range check %s, past_range_zero=%d\n",
+                      bad, per_dword ? "per dword" : "NOT per dword", (int)beyond_zero);
+        rep += line;
+        if (bad || !per_dword || !beyond_zero) all_ok = false;
+        (void)hipFree(d);
+        (void)hipFree(o);
     }
 
     // ---- MFMA operand / accumulator layout for the four families

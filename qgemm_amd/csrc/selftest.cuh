@@ -44,6 +44,16 @@ __global__ void __launch_bounds__(64) probe_mfma_kernel(const char *x, const cha
 #endif
 }
 
+// Lane l loads 8 bytes at byte offset 4 * l of a raw buffer of `range` bytes (an a_scale row with an odd number of K
+// blocks starts every other row at such an offset, and the last pair of the last row straddles the end of the range).
+__global__ void __launch_bounds__(64) probe_b64_load_kernel(const float *src, uint32_t range, int *out) {
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(src, range);
+    const int lane = threadIdx.x;
+    const v2i v = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(r, lane * 4, 0, 0));
+    out[2 * lane] = v[0];
+    out[2 * lane + 1] = v[1];
+}
+
 // Every workgroup records which XCD (XCC_ID hardware register) and CU it ran on.
 __global__ void __launch_bounds__(64) probe_xcc_kernel(uint32_t *out) {
 #if defined(__HIP_DEVICE_COMPILE__)

@@ -105,9 +105,9 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 1536, 7168, 2048) == "192x256_w2x4_solo8_ks"
     assert plan(Q.DT_BF16, 0, 0, 8192, 4096, 4096) == "256x256_w2x2_solo"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "256x256_w2x2_solo"  # config 3
-    # config 4: the twin of the 8-wave kernel that reads a_scale as this layout passes it (56 K blocks per row: even)
+    # config 4: the twin of the 8-wave kernel that reads a_scale as this layout passes it (any number of K blocks per row)
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8_ks+192x256_w2x4_solo8_ks"    # config 4: 14 row bands on 256 x 256, the 2560 rows below on 192 x 256
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168 - 128) == "256x256_w2x4_solo8+192x256_w2x4_solo8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168 - 128) == "256x256_w2x4_solo8_ks+192x256_w2x4_solo8_ks"
     # config 5: the skinny-M kernel (K split over the eight waves of a workgroup)
     for m, name in ((16, "skinny_16x32_k8"), (64, "skinny_64x32_k8"), (128, "skinny_64x64_k8")):
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
@@ -174,8 +174,8 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 2, 1024, 1024, 1024).startswith("transpose+")   # no K-major int8 family
     # K bytes not a multiple of 16: the any-shape kernel; whole 16-byte chunks with a partial last K step: the MFMA kernels
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 100, 100, 100) == "strided_any_shape"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7200) == "256x256_w2x4_solo8+192x256_w2x4_solo8"       # (57 K blocks: no twin)
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7216) == "256x256_w2x4_solo8+192x256_w2x4_solo8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7200) == "256x256_w2x4_solo8_ks+192x256_w2x4_solo8_ks"       # (57 K blocks)
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7216) == "256x256_w2x4_solo8_ks+192x256_w2x4_solo8_ks"
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4000) == plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4096)
     assert plan(Q.DT_BF16, 0, 0, 1024, 1024, 1000) == plan(Q.DT_BF16, 0, 0, 1024, 1024, 1024)
     assert plan(Q.DT_BF16, 0, 0, 1024, 1024, 1004) == "strided_any_shape"

@@ -180,14 +180,15 @@ def test_fp8_block_scaled_power_of_two_scales_bit_exact(variant, shape):
     assert np.array_equal(host(c), ref), Q.last_config()
 
 
-@pytest.mark.parametrize("case", [(512, 512, 1024, 0, True), (300, 520, 768, 0, True), (256, 256, 1536, 2, True),
-                                  (256, 256, 1280, 2, False), (256, 256, 384, 0, False), (512, 256, 7168, 0, True)])
+@pytest.mark.parametrize("case", [(512, 512, 1024, 0), (300, 520, 768, 0), (256, 256, 1536, 2),
+                                  (256, 256, 1280, 2), (256, 256, 384, 0), (512, 256, 7168, 0), (300, 256, 7296, 3)])
 def test_fp8_block_scaled_k_contiguous_scale_twin(case):
-    """The block-scaled 8-wave kernel reads a_scale as QGEMM_LAYOUT_K_CONTIGUOUS passes it (two K blocks per load)
-    when every row holds an even number of K blocks and every K slice an even number of steps, and falls back to
-    a rows-contiguous copy otherwise; bit-exact either way on small integers and power-of-two scales, so a scale
+    """The block-scaled 8-wave kernel reads a_scale as QGEMM_LAYOUT_K_CONTIGUOUS passes it, two K blocks per 8-byte
+    load, whatever the number of K blocks per row (an odd one puts every other row at a 4-byte aligned address and
+    lets the pair behind a row's last block reach into the next row, or past the end of the array, where the buffer
+    range check returns zero for it) and per K slice; bit-exact on small integers and power-of-two scales, so a scale
     taken from the wrong K block or row cannot pass."""
-    M, N, K, split, twin = case
+    M, N, K, split = case
     say("fp8 block, K-contiguous a_scale", case)
     rng = np.random.default_rng(17)
     a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
@@ -199,14 +200,15 @@ def test_fp8_block_scaled_k_contiguous_scale_twin(case):
     Q.set_option("force_split", split)
     c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), dev(as_), dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
-    assert ("solo8_ks" in Q.last_config()) == twin, Q.last_config()
+    assert "solo8_ks" in Q.last_config(), Q.last_config()
     assert np.array_equal(host(c), ref), Q.last_config()
-    # scales whose rows are not 8-byte aligned: the copy again
-    as_off = torch.zeros(as_.size + 1, dtype=torch.float32, device="cuda")
-    as_off[1:] = dev(as_).flatten()
+    # scales that start at a 4-byte aligned address, with NaNs in front of and behind the array: nothing outside it
+    # may reach a result
+    as_off = torch.full((as_.size + 2,), float("nan"), dtype=torch.float32, device="cuda")
+    as_off[1:-1] = dev(as_).flatten()
     c.zero_()
-    Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), as_off[1:], dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
-    assert "solo8_ks" not in Q.last_config()
+    Q.scaled_gemm(fp8_tensor(R.encode_fp8(a)), fp8_tensor(R.encode_fp8(b)), as_off[1:-1], dev(bs), c, M, N, K, Q.SCALE_BLOCK128)
+    assert "solo8_ks" in Q.last_config(), Q.last_config()
     assert np.array_equal(host(c), ref), Q.last_config()
 
 

@@ -116,13 +116,13 @@ def test_static_scratch_entry_refuses_what_does_not_fit():
     # ... and the room for a transposed a_scale: 131072 rows x 72 K blocks of floats = 36 MiB
     say("no-alloc entry: too large, transposed a_scale")
     M, N, K = 131072, 128, 72 * 128 + 128
-    KB = K // 128                                      # odd: the kernels want a_scale rows-contiguous, through a copy
+    KB = K // 128                                      # 73: the row with copying waves fetches four K blocks a copy or wants a_scale rows-contiguous, through a copy
     a = torch.zeros((M, K), dtype=torch.uint8, device="cuda")
     b = torch.zeros((N, K), dtype=torch.uint8, device="cuda")
     sa = torch.ones((M, KB), dtype=torch.float32, device="cuda")
     sb = torch.ones((1, KB), dtype=torch.float32, device="cuda")
     cb = torch.full((M, N), 3.0, dtype=torch.bfloat16, device="cuda")
-    Q.force_config("256x256_w2x4_solo8")
+    Q.force_config("256x128_w2x2_cw")
     try:
         assert _call(True, Q.DT_F8E4M3, Q.SCALE_BLOCK128, Q.LAYOUT_K_CONTIGUOUS, a, b, sa, sb, cb, M, N, K, 1) == 10
     finally:
