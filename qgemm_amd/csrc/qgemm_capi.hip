@@ -64,6 +64,7 @@ struct Context {
     long k_rot = -1;            // -1: rotated K start for at most 256 rows (see plan_nt), 0: never, n: steps per column tile
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long stagger_groups = 8;    // groups the workgroups of the first round start in
+    long c_plain = -1;          // -1: the library decides; 0 / 1: non-temporal / ordinary stores for C
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch;
                                 // 2: always where the geometry allows it, whatever the estimate says (for measurements)
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes; 2: never
@@ -690,6 +691,13 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
         // f32 128 us without, 139 us with)
         const bool spread = v.bm == 256 && v.bn == 256 && ob == 4 && pl.tiles >= 3 * (size_t)g_ctx.num_cus && a.ksteps >= 32;
         a.stagger = g_ctx.stagger >= 0 ? (uint32_t)g_ctx.stagger : (spread ? 1u : 0u);
+        // 4-byte C from 256 x 256 tiles: ordinary stores up to two rounds of tiles, non-temporal ones (and the staggered
+        // start) from three on.  int8 to f32, ordinary against non-temporal, interleaved: 4096^3 59.1 against 61.1 us,
+        // 4096 x 8192 x 4096 (two rounds) 114.2 against 124.0, 6144 x 8192 x 4096 (three) 165.6 against 169.9 with the
+        // stagger, 8192^3 (four) 399.4 against 386.9; 2-byte C and every other tile are 1 - 6 % slower with ordinary
+        // stores (the row with copying waves, 192 x 256, the K-group rows, 64 x 128).
+        a.c_plain = g_ctx.c_plain >= 0 ? (int)g_ctx.c_plain
+                                       : (v.bm == 256 && v.bn == 256 && ob == 4 && pl.tiles < 3 * (size_t)g_ctx.num_cus);
         a.stagger_wgs = (uint32_t)g_ctx.num_cus;
         a.stagger_groups = (uint32_t)std::max<long>(1, std::min<long>(32, g_ctx.stagger_groups));
         hipError_t e = v.launch(a, (uint32_t)pl.tiles, stream);
@@ -982,6 +990,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "kmajor")) g_ctx.kmajor = value;
     else if (!std::strcmp(key, "stagger")) g_ctx.stagger = value;
     else if (!std::strcmp(key, "stagger_groups")) g_ctx.stagger_groups = value;
+    else if (!std::strcmp(key, "c_plain")) g_ctx.c_plain = value;
     else if (!std::strcmp(key, "k_rot")) g_ctx.k_rot = value;
     else if (!std::strcmp(key, "as_groups")) g_ctx.as_groups = value;
 #if QGEMM_DEBUG_BUILD
