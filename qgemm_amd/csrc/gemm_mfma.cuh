@@ -70,6 +70,7 @@ struct GemmArgs {
     int per_matrix_scale; // multiply by as[0]*bs[0] in the epilogue
     int vec_store;        // 0: scalar stores; 1: C and ldc allow 4-element vector stores; 2: also 16-byte row pieces
     int c_plain;          // ordinary instead of non-temporal stores for C (run_nt: launches of at most one round of tiles)
+    int b_stream;         // B is read once by the launch (one or two row tiles): its copies carry the streaming hint
     uint32_t k_rot;                  // simple pipeline and skinny-M kernel: the workgroups of column tile i start their K loops (i * k_rot) % nk steps in (0: at 0)
     uint32_t stagger, stagger_wgs;   // the first stagger_wgs workgroups start (id / 8 % stagger_groups) * stagger microseconds late (0: off)
     uint32_t stagger_groups;
@@ -409,8 +410,11 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
 #pragma unroll
         for (int i = 0; i < C::LPT; ++i) {
             lds_void *dst = (lds_void *)(stage + (wave + i * C::NW) * 1024);
+            // (B read once by the launch, i.e. streamed out of memory: its copies carry the streaming hint)
             if (i < LPT_A0)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, va, load_soff(i, kt), 0, 0);
+            else if (p.b_stream)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, load_soff(i, kt), 0, 2);
             else
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, load_soff(i, kt), 0, 0);
         }
@@ -1055,7 +1059,10 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         if (2 * j < C::RBA)
                             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, va, soff_k2(C::KMA, blk, p.lda, kt), 0, 0);
                         else
-                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 0);
+                            if (p.b_stream)      // (B read once by the launch: the streaming hint, as in issue_stage)
+                                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 2);
+                            else
+                                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 0);
                     }
                     if constexpr (C::BLOCK_SCALE) {
                         if (!p.as_groups) {

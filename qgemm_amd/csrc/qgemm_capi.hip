@@ -65,6 +65,7 @@ struct Context {
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long stagger_groups = 8;    // groups the workgroups of the first round start in
     long c_plain = -1;          // -1: the library decides; 0 / 1: non-temporal / ordinary stores for C
+    long b_stream = -1;         // -1: the library decides; 0 / 1: B copies of the skinny-M kernel without / with the streaming hint
     long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch;
                                 // 2: always where the geometry allows it, whatever the estimate says (for measurements)
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes; 2: never
@@ -612,6 +613,7 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
     a.bs_ns = q.bs_ns;
     a.bs_ks = q.bs_ks;
     a.nb_max = (uint32_t)((q.N + 127) / 128 - 1);
+    a.b_stream = g_ctx.b_stream >= 0 ? (int)g_ctx.b_stream : (a.tiles_m == 1);
     pl.tiles = (size_t)a.tiles_m * a.tiles_n;
     if (pl.tiles * 64 >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
 
@@ -991,6 +993,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "stagger")) g_ctx.stagger = value;
     else if (!std::strcmp(key, "stagger_groups")) g_ctx.stagger_groups = value;
     else if (!std::strcmp(key, "c_plain")) g_ctx.c_plain = value;
+    else if (!std::strcmp(key, "b_stream")) g_ctx.b_stream = value;
     else if (!std::strcmp(key, "k_rot")) g_ctx.k_rot = value;
     else if (!std::strcmp(key, "as_groups")) g_ctx.as_groups = value;
 #if QGEMM_DEBUG_BUILD
