@@ -238,10 +238,16 @@ def main():
                 us_rot = _graph_time([mk(bq, sbq) for (bq, sbq) in b5s])
                 us_res = _graph_time([mk(*b5s[0])] * nbuf)
                 us_rot_load = _graph_time([mk(bq, sbq) for (bq, sbq) in b5s], load_ms=LOAD_MS)
+                # option b_stream = 1: the streaming hint on the copies of B, which the library puts on by itself only
+                # for a B of 64 MiB or more (a caller that loops over one small B would find it in the memory-side cache)
+                Q.set_option("b_stream", 1)
+                us_rot_stream = _graph_time([mk(bq, sbq) for (bq, sbq) in b5s])
+                Q.set_option("b_stream", -1)
                 nbytes = n5 * k5 + m5 * k5 + m5 * n5 * c5.element_size()
                 extra["cfg5_%s_skinny_M%d" % (fam, m5)] = {
                     "us_per_launch_rotated": us_rot, "us_per_launch_resident": us_res,
                     "us_per_launch_rotated_behind_%d_ms_of_replays" % LOAD_MS: us_rot_load,
+                    "us_per_launch_rotated_with_option_b_stream": us_rot_stream,
                     "GBps": nbytes / us_rot / 1e3, "frac_of_hbm_peak": nbytes / us_rot / 1e3 / PEAK_HBM_GBS,
                     "GBps_resident": nbytes / us_res / 1e3, "tflops": 2.0 * m5 * n5 * k5 / us_rot / 1e6,
                     "algorithmic_bytes": nbytes, "kernel": Q.last_config()}
