@@ -239,7 +239,7 @@ def main():
                 us_res = _graph_time([mk(*b5s[0])] * nbuf)
                 us_rot_load = _graph_time([mk(bq, sbq) for (bq, sbq) in b5s], load_ms=LOAD_MS)
                 # option b_stream = 1: the streaming hint on the copies of B, which the library puts on by itself only
-                # for a B of 64 MiB or more (a caller that loops over one small B would find it in the memory-side cache)
+                # for a B of 32 MiB or more (a caller that loops over one small B would find it in the memory-side cache)
                 Q.set_option("b_stream", 1)
                 us_rot_stream = _graph_time([mk(bq, sbq) for (bq, sbq) in b5s])
                 Q.set_option("b_stream", -1)

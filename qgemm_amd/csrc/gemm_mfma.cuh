@@ -1048,7 +1048,8 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                     if (kmajor) return (k * C::KE + (blk % BPP) * 16) * ld + (blk / BPP) * 128;
                     return blk * 16 * ld + k * C::BKB;
                 };
-                auto issue_stage_k2 = [&](int kt) {
+                auto issue_stage_k2 = [&](int kt, auto nt_tag) {          // (nt_tag: B's copies with the streaming hint)
+                    constexpr bool B_NT = decltype(nt_tag)::value;
                     char *stage = smem + (kt % NS) * C::STAGE_BYTES + pw * 1024;
                     const bool tl = kpos(kt) == kt_tail;
                     const uint32_t va = tl ? voff_a_t : voff_a, vb = tl ? voff_b_t : voff_b;
@@ -1059,10 +1060,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         if (2 * j < C::RBA)
                             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, va, soff_k2(C::KMA, blk, p.lda, kt), 0, 0);
                         else
-                            if (p.b_stream)      // (B read once by the launch: the streaming hint, as in issue_stage)
-                                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 2);
-                            else
-                                __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, 0);
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, vb, soff_k2(C::KMB, blk - C::RBA, p.ldb, kt), 0, B_NT ? 2 : 0);
                     }
                     if constexpr (C::BLOCK_SCALE) {
                         if (!p.as_groups) {
@@ -1079,23 +1077,29 @@ __global__ void __launch_bounds__(C::THREADS) gemm_nt_kernel(const GemmArgs p) {
                         }
                     }
                 };
+                // (the loop of a copying wave exists twice, with and without the streaming hint on B's copies: chosen per
+                // copy inside one loop the branch cost these waves 2 - 4 %)
+                auto copy_loop = [&](auto nt_tag) {
 #pragma unroll
-                for (int j = 0; j < NS - 1; ++j)
-                    if (j < nk) {
-                        issue_scale_group(j);
-                        issue_stage_k2(j);
+                    for (int j = 0; j < NS - 1; ++j)
+                        if (j < nk) {
+                            issue_scale_group(j);
+                            issue_stage_k2(j, nt_tag);
+                        }
+                    const bool counted = !C::BLOCK_SCALE || !p.as_groups;       // the scale copies are among the CPS of a stage
+                    for (int ph = 0; ph <= nk; ++ph) {
+                        if (ph + NS - 2 >= nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
+                        else if (counted) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * CPS));
+                        else __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * NPC));
+                        phase_barrier();
+                        if (ph + NS - 1 < nk) {
+                            issue_scale_group(ph + NS - 1);
+                            issue_stage_k2(ph + NS - 1, nt_tag);
+                        }
                     }
-                const bool counted = !C::BLOCK_SCALE || !p.as_groups;       // the scale copies are among the CPS of a stage
-                for (int ph = 0; ph <= nk; ++ph) {
-                    if (ph + NS - 2 >= nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));      // near the end of K fewer are in flight
-                    else if (counted) __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * CPS));
-                    else __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * NPC));
-                    phase_barrier();
-                    if (ph + NS - 1 < nk) {
-                        issue_scale_group(ph + NS - 1);
-                        issue_stage_k2(ph + NS - 1);
-                    }
-                }
+                };
+                if (p.b_stream) copy_loop(std::integral_constant<bool, true>{});
+                else copy_loop(std::integral_constant<bool, false>{});
             } else {
                 v4i fa[C::TM][2], fb[C::TN][2];
                 auto read_stage = [&](int mine) {

@@ -613,14 +613,15 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
     a.bs_ns = q.bs_ns;
     a.bs_ks = q.bs_ks;
     a.nb_max = (uint32_t)((q.N + 127) / 128 - 1);
-    // Copies of B with the streaming hint: where the launch reads B once (one row tile) and B is too large to be found
-    // in the 256 MB memory-side cache by the next call (64 MiB or more).  With B out of memory the hint is worth 2 - 12 %
+    // Copies of B with the streaming hint: where the launch reads B once (one row tile) and B is unlikely to be found in
+    // the 256 MB memory-side cache by the next call (32 MiB or more: beyond what the L2s hold together).  With B out of
+    // memory the hint is worth 2 - 12 %
     // (16 x 28672 x 8192 fp8 44.6 -> 40.2 us, 1 x 8192 x 8192 14.8 -> 13.0, 16 / 64 x 7168 x 2048 5.67 / 6.96 -> 5.40 / 6.75);
     // a caller who loops over one small B that sits in that cache loses 14 - 30 % with it (the same shapes with one B:
     // 3.56 / 5.04 -> 4.61 / 5.73), and with two row tiles sharing a strip of B it costs up to 8 %.  Option b_stream = 1
     // puts it on for every launch with one row tile: for callers whose weights do not stay in the cache between calls.
     a.b_stream = g_ctx.b_stream >= 0 ? (int)(g_ctx.b_stream && a.tiles_m == 1)
-                                     : (a.tiles_m == 1 && q.N * q.Kbytes >= ((size_t)64 << 20));
+                                     : (a.tiles_m == 1 && q.N * q.Kbytes >= ((size_t)32 << 20));
     pl.tiles = (size_t)a.tiles_m * a.tiles_n;
     if (pl.tiles * 64 >= ((size_t)1 << 31)) return QGEMM_ERR_TOO_LARGE;
 
