@@ -114,7 +114,7 @@ def one_shape(Q, torch, dev, spec, launches):
         Q.set_option("dbg_ptr", 0)
     except Q.QgemmError:
         return out
-    if "+" in out["kernel"] or "skinny" in out["kernel"] or "splitk" in out["kernel"]:
+    if "+" in out["kernel"] or "|" in out["kernel"] or "skinny" in out["kernel"] or "splitk" in out["kernel"]:
         return out
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     slots = 1 << 16                                          # workgroups x waves of any variant on any shape tried here

@@ -66,8 +66,9 @@ struct Context {
     long stagger_groups = 8;    // groups the workgroups of the first round start in
     long c_plain = -1;          // -1: the library decides; 0 / 1: non-temporal / ordinary stores for C
     long b_stream = -1;         // -1: the library decides; 0 / 1: B copies of the skinny-M kernel without / with the streaming hint
-    long row_split = 1;         // 0: never run the rows of a last, mostly empty round of 256 x 256 tiles as a second launch;
-                                // 2: always where the geometry allows it, whatever the estimate says (for measurements)
+    long row_split = 1;         // 0: never run the rows (or columns) of a last, mostly empty round of 256 x 256 tiles as a second launch;
+                                // 2 / 3: the rows / the columns always where the geometry allows it, whatever the estimate says
+                                // (for measurements)
     long kmajor = 1;            // 0: K-major operands (NN, reference fp8 layout) always go through the transposes; 2: never
                                 // where a K-major kernel fits the shape (for measurements and tests)
     std::string last_config;
@@ -338,7 +339,9 @@ int choose_by_cost(const Variant *tab, int count, size_t M, size_t N, size_t kst
 int choose_tile(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int kmaj, int cus,
                 bool may_split, uint32_t *nsplit_out);
 size_t rows_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus,
-                            double t_single, double *t_split = nullptr);
+                            double t_single, double *t_split = nullptr, size_t *padding = nullptr);
+size_t cols_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus,
+                            double t_single, double *t_split = nullptr, size_t *padding = nullptr, bool whatever_the_estimate = false);
 
 // The skinny-M kernel (gemm_skinny.cuh: the K split inside the workgroup, eight waves each on every eighth K step)
 // takes over from the narrow simple-pipeline tiles where it is faster: one row tile (M <= 128), a strip of 32
@@ -501,9 +504,12 @@ bool kmajor_problem_ok(NtProblem q, int kmaj, size_t lda_bytes, size_t ldb_bytes
     if (q.M > 128 && may_split) {                    // (the K-contiguous route may split the rows into two launches)
         double t_single = 0, t_split = 0;
         uint32_t ns1 = 0;
-        if (choose_by_cost(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, false, &ns1, &t_single) >= 0 &&
-            rows_for_full_rounds(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, t_single, &t_split) && t_split < t_nt)
-            t_nt = t_split;
+        if (choose_by_cost(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, false, &ns1, &t_single) >= 0) {
+            if (rows_for_full_rounds(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, t_single, &t_split) && t_split < t_nt)
+                t_nt = t_split;
+            if (cols_for_full_rounds(tab, count, q.M, q.N, ksteps, q.block, g_ctx.num_cus, t_single, &t_split) && t_split < t_nt)
+                t_nt = t_split;
+        }
     }
     const double kbytes = (double)q.Kbytes;         // K * element size
     t_nt += 1.0;                                     // a transpose launch per operand: 4 us and the matrix read and written
@@ -520,8 +526,15 @@ struct Plan {
     // Row split: this plan covers rows [0, m_main) of the problem and `rest` the rows below, as a second launch
     // with a tile of its own (m_main = 0: no split, the plan covers everything).
     size_t m_main = 0;
+    // Column split, the same along N: columns [0, n_main) here, the columns to the right in `rest` (never both splits)
+    size_t n_main = 0;
     std::unique_ptr<Plan> rest;
 };
+
+// elements the tiles of a launch compute beyond the M x N asked for
+size_t padded_area(size_t bm, size_t bn, size_t M, size_t N) {
+    return ((M + bm - 1) / bm * bm) * ((N + bn - 1) / bn * bn) - M * N;
+}
 
 // Rows of the problem that 256 x 256 tiles should take when such tiles do not fill the last round of CUs.
 // 576 tiles on 256 CUs are 2.25 rounds and cost three: the rows of the two full rounds go to one launch, and the
@@ -533,7 +546,7 @@ struct Plan {
 // second) is not at least 2.5 % below the estimate t_single of the one (config 4 with block scales: estimate
 // 160.5 against 164.8 us, 2.6 %; measured 170.9 - 172.5 against 175.1 - 176.9 us in three interleaved runs).
 size_t rows_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus,
-                            double t_single, double *t_split) {
+                            double t_single, double *t_split, size_t *padding) {
     if (!g_ctx.row_split) return 0;
     const size_t tn = (N + 255) / 256, tiles = ((M + 255) / 256) * tn, full = tiles / cus;
     if (full == 0 || tiles % cus == 0) return 0;
@@ -543,14 +556,41 @@ size_t rows_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, s
     double t_main = 0, t_rest = 0;
     const int vm = choose_by_cost(tab, count, m_main, N, ksteps, block, cus, false, &ns, &t_main);
     if (vm < 0 || tab[vm].bm != 256 || tab[vm].bn != 256) return 0;
+    size_t pad = padded_area(256, 256, m_main, N);
     if (M - m_main > 128) {
-        if (choose_by_cost(tab, count, M - m_main, N, ksteps, block, cus, false, &ns, &t_rest) < 0) return 0;
+        const int vr = choose_by_cost(tab, count, M - m_main, N, ksteps, block, cus, false, &ns, &t_rest);
+        if (vr < 0) return 0;
+        pad += padded_area(tab[vr].bm, tab[vr].bn, M - m_main, N);
     } else {
         t_rest = 5.0 + (double)N * ksteps * 128.0 / 4.0e6;      // B streamed once, about 4 TB/s
     }
     if (t_split) *t_split = t_main + t_rest + 6.0;
+    if (padding) *padding = pad;
     if (g_ctx.row_split == 2) return m_main;
     return t_main + t_rest + 6.0 < 0.975 * t_single ? m_main : 0;
+}
+
+// The same along N, for shapes whose row tiles do not divide the full rounds but whose column tiles do:
+// 4096 x 14336 x 4096 is 16 x 56 tiles, 3.5 rounds; 13 of its 16 row tiles are 2.84 rounds and still cost three, while
+// 48 of its 56 column tiles are exactly three, and the 4096 x 2048 to their right fill a round of smaller tiles.
+// Returns the columns of the first launch (a multiple of 256, so the right part starts on a 128-block of b_scale).
+size_t cols_for_full_rounds(const Variant *tab, int count, size_t M, size_t N, size_t ksteps, bool block, int cus,
+                            double t_single, double *t_split, size_t *padding, bool whatever_the_estimate) {
+    if (!g_ctx.row_split) return 0;
+    const size_t tm = (M + 255) / 256, tiles = tm * ((N + 255) / 256), full = tiles / cus;
+    if (full == 0 || tiles % cus == 0) return 0;
+    const size_t n_main = (full * cus / tm) * 256;
+    if (n_main == 0 || n_main >= N) return 0;
+    uint32_t ns = 0;
+    double t_main = 0, t_rest = 0;
+    const int vm = choose_by_cost(tab, count, M, n_main, ksteps, block, cus, false, &ns, &t_main);
+    if (vm < 0 || tab[vm].bm != 256 || tab[vm].bn != 256) return 0;
+    const int vr = choose_by_cost(tab, count, M, N - n_main, ksteps, block, cus, false, &ns, &t_rest);
+    if (vr < 0) return 0;
+    if (t_split) *t_split = t_main + t_rest + 6.0;
+    if (padding) *padding = padded_area(256, 256, M, n_main) + padded_area(tab[vr].bm, tab[vr].bn, M, N - n_main);
+    if (g_ctx.row_split == 3 || whatever_the_estimate) return n_main;
+    return t_main + t_rest + 6.0 < 0.975 * t_single ? n_main : 0;
 }
 
 int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
@@ -565,17 +605,39 @@ int plan_nt(const NtProblem &q, Plan &pl, bool may_split_rows = true) {
         double t_single = 0;
         const int ci = choose_by_cost(tab, count, q.M, q.N, ksteps_of(q), q.block, g_ctx.num_cus, false, &ns, &t_single);
         if (ci >= 0 && tab[ci].bm == tab[vi].bm && tab[ci].bn == tab[vi].bn && tab[ci].kgroups == tab[vi].kgroups) {
-            const size_t m_main = rows_for_full_rounds(tab, count, q.M, q.N, ksteps_of(q), q.block, g_ctx.num_cus, t_single);
-            if (m_main) {
+            double t_rows = 0, t_cols = 0;
+            size_t pad_rows = 0, pad_cols = 0;
+            size_t m_main = rows_for_full_rounds(tab, count, q.M, q.N, ksteps_of(q), q.block, g_ctx.num_cus, t_single, &t_rows, &pad_rows);
+            size_t n_main = g_ctx.row_split == 2 ? 0
+                                : cols_for_full_rounds(tab, count, q.M, q.N, ksteps_of(q), q.block, g_ctx.num_cus, t_single, &t_cols, &pad_cols, m_main != 0);
+            // The columns by themselves where they are estimated at least 2.5 % ahead of the single launch, as the rows are.
+            // Where the rows pass that test, the columns take their place if they are estimated 5 % faster, or no more
+            // than 5 % slower with tiles that compute less beyond the matrix: the estimate prices tiles, not the rows in
+            // them that count, and a full round of 256 tiles more than one of 252.  Config 4 is 14 row bands of 256 x 256
+            // tiles and 2560 rows below on 192 x 256 ones, the last band of which is two thirds padding, or 10 column bands
+            // and 2048 columns to the right that 32 x 8 such tiles cover exactly: 172.8 against 170.8 us, and 143.0
+            // against 139.8 with per-matrix scales.  (Measured, the two are never further apart than 2.3 %.)
+            if (g_ctx.row_split == 3) m_main = 0;
+            if (m_main && n_main) {
+                const bool cols = t_cols < 0.95 * t_rows || (t_cols <= 1.05 * t_rows && pad_cols < pad_rows);
+                (cols ? m_main : n_main) = 0;
+            }
+            if (m_main || n_main) {
                 NtProblem q_main = q, q_rest = q;
-                q_main.M = m_main;
-                q_rest.M = q.M - m_main;
+                if (m_main) {
+                    q_main.M = m_main;
+                    q_rest.M = q.M - m_main;
+                } else {
+                    q_main.N = n_main;
+                    q_rest.N = q.N - n_main;
+                }
                 int st = plan_nt(q_main, pl, false);
                 if (st != QGEMM_OK) return st;
                 pl.rest.reset(new Plan());
                 st = plan_nt(q_rest, *pl.rest, false);
                 if (st != QGEMM_OK) return st;
                 pl.m_main = m_main;
+                pl.n_main = n_main;
                 pl.split_bytes = std::max(pl.split_bytes, pl.rest->split_bytes);     // one after the other on the stream
                 return QGEMM_OK;
             }
@@ -651,16 +713,25 @@ int run_nt(const NtProblem &q, Plan &pl, void *split_ws, hipStream_t stream) {
     if (pl.rest) {
         // rows [0, m_main) with this plan, the rows below with the other: operands, scales and C move down m_main rows
         NtProblem q_main = q, q_rest = q;
-        q_main.M = pl.m_main;
-        q_rest.M = q.M - pl.m_main;
-        q_rest.A = (const char *)q.A + pl.m_main * q.lda_bytes;            // (K-contiguous operands only: plan_nt)
-        q_rest.C = (char *)q.C + pl.m_main * q.ldc * dtype_bytes(q.out_dtype);
-        if (q.block && q.as) q_rest.as = q.as + pl.m_main * q.as_ms;
+        if (pl.m_main) {
+            q_main.M = pl.m_main;
+            q_rest.M = q.M - pl.m_main;
+            q_rest.A = (const char *)q.A + pl.m_main * q.lda_bytes;            // (K-contiguous operands only: plan_nt)
+            q_rest.C = (char *)q.C + pl.m_main * q.ldc * dtype_bytes(q.out_dtype);
+            if (q.block && q.as) q_rest.as = q.as + pl.m_main * q.as_ms;
+        } else {
+            // columns [0, n_main) with this plan, the columns to the right with the other: B, its scale blocks and C move
+            q_main.N = pl.n_main;
+            q_rest.N = q.N - pl.n_main;
+            q_rest.B = (const char *)q.B + pl.n_main * q.ldb_bytes;
+            q_rest.C = (char *)q.C + pl.n_main * dtype_bytes(q.out_dtype);
+            if (q.block && q.bs) q_rest.bs = q.bs + (pl.n_main / 128) * q.bs_ns;
+        }
         std::unique_ptr<Plan> rest = std::move(pl.rest);
         int st = run_nt(q_main, pl, split_ws, stream);
         const std::string first = g_ctx.last_config;
         if (st == QGEMM_OK) st = run_nt(q_rest, *rest, split_ws, stream);
-        g_ctx.last_config = first + "+" + g_ctx.last_config;
+        g_ctx.last_config = first + (pl.m_main ? "+" : "|") + g_ctx.last_config;        // rows + rows below, columns | columns to the right
         pl.rest = std::move(rest);
         return st;
     }
@@ -1105,7 +1176,7 @@ QGEMM_EXPORT int qgemm_plan(int in_dtype, int scale_mode, int k_major, size_t M,
     name += std::string(pl.v->name) + kmaj_suffix(q.kmaj);
     if (pl.a.nsplit > 1) name += "_splitk" + std::to_string(pl.a.nsplit);
     if (pl.rest) {
-        name += "+" + std::string(pl.rest->v->name);
+        name += (pl.m_main ? "+" : "|") + std::string(pl.rest->v->name);
         if (pl.rest->a.nsplit > 1) name += "_splitk" + std::to_string(pl.rest->a.nsplit);
     }
     std::snprintf(buf, buflen, "%s", name.c_str());

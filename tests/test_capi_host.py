@@ -106,8 +106,9 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_BF16, 0, 0, 8192, 4096, 4096) == "256x256_w2x2_solo"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 8192, 8192, 8192) == "256x256_w2x2_solo"  # config 3
     # config 4: the twin of the 8-wave kernel that reads a_scale as this layout passes it (any number of K blocks per row)
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8_ks+192x256_w2x4_solo8_ks"    # config 4: 14 row bands on 256 x 256, the 2560 rows below on 192 x 256
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168 - 128) == "256x256_w2x4_solo8_ks+192x256_w2x4_solo8_ks"
+    # config 4: 10 column bands on 256 x 256 tiles (240 of them), the 2048 columns to the right on 32 x 8 tiles of 192 x 256
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168) == "256x256_w2x4_solo8_ks|192x256_w2x4_solo8_ks"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7168 - 128) == "256x256_w2x4_solo8_ks|192x256_w2x4_solo8_ks"
     # config 5: the skinny-M kernel (K split over the eight waves of a workgroup)
     for m, name in ((16, "skinny_16x32_k8"), (64, "skinny_64x32_k8"), (128, "skinny_64x64_k8")):
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
@@ -155,7 +156,17 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 5000, 4096, 7168) == "256x256_w2x2_solo+128x128_w2x2_k2"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 7000, 7168, 2048) == "256x256_w2x2_solo+skinny_64x64_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 7000, 7168, 2048) == "256x256_w2x4_solo8_ks+skinny_64x64_k8"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 4096, 14336, 4096) == "256x256_w2x2_solo"     # 3.5 rounds: no gain
+    # ... or its columns ("|"), where those divide the full rounds and the rows do not: 16 x 56 tiles are 3.5 rounds, 48
+    # column bands exactly three, and the 4096 x 2048 to their right one round of 256 x 128 tiles (176 -> 172 us)
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 4096, 14336, 4096) == "256x256_w2x2_solo|256x128_w2x2_cw"
+    assert plan(Q.DT_BF16, 0, 0, 8192, 4608, 4096) == "256x256_w2x2_solo|128x128_w2x2_k2"
+    Q.set_option("row_split", 2)            # (2 / 3: the rows / the columns wherever the geometry allows)
+    try:
+        assert plan(Q.DT_BF16, 0, 0, 8192, 4608, 4096) == "256x256_w2x2_solo+256x128_w2x2_cw"
+        Q.set_option("row_split", 3)
+        assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 6144, 6144, 6144) == "256x256_w2x2_solo|256x128_w2x2_cw"
+    finally:
+        Q.set_option("row_split", 1)
     Q.set_option("row_split", 0)
     try:
         # (one launch: 768 tiles of 192 x 256 are three full rounds, 166 us against 187 on 256 x 256 tiles)
@@ -165,7 +176,7 @@ def test_plan_names_the_kernel_without_a_device():
     # operands stored K-major: read as stored where that is cheaper than transposing, else transposed first
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 2048, 2048, 2048) == "128x128_w2x2_k2_tn"
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 4096, 2048, 2048) == "256x128_w2x2_cw_tn"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 6144, 4608, 7168) == "transpose+256x256_w2x4_solo8+192x256_w2x4_solo8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 3, 6144, 4608, 7168) == "transpose+256x256_w2x4_solo8|192x256_w2x4_solo8"
     assert plan(Q.DT_BF16, 0, 2, 1024, 1024, 1024) == "64x128_w1x4_k2_nn"
     assert plan(Q.DT_BF16, 0, 2, 8192, 8192, 8192) == "transpose+256x256_w2x2_solo"
     # large shapes whose transposes are a sizeable part: as stored, on the K-major 256 x 128 row with copying waves
@@ -174,8 +185,8 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 2, 1024, 1024, 1024).startswith("transpose+")   # no K-major int8 family
     # K bytes not a multiple of 16: the any-shape kernel; whole 16-byte chunks with a partial last K step: the MFMA kernels
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 100, 100, 100) == "strided_any_shape"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7200) == "256x256_w2x4_solo8_ks+192x256_w2x4_solo8_ks"       # (57 K blocks)
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7216) == "256x256_w2x4_solo8_ks+192x256_w2x4_solo8_ks"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7200) == "256x256_w2x4_solo8_ks|192x256_w2x4_solo8_ks"       # (57 K blocks)
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 6144, 4608, 7216) == "256x256_w2x4_solo8_ks|192x256_w2x4_solo8_ks"
     assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4000) == plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, 4096, 4096, 4096)
     assert plan(Q.DT_BF16, 0, 0, 1024, 1024, 1000) == plan(Q.DT_BF16, 0, 0, 1024, 1024, 1024)
     assert plan(Q.DT_BF16, 0, 0, 1024, 1024, 1004) == "strided_any_shape"

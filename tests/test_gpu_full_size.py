@@ -289,6 +289,67 @@ def test_row_split_of_a_partly_empty_last_round():
     assert_close(host(c16)[rows], R.gemm_f32acc(R.decode_bf16(ha[rows]), R.decode_bf16(hb)), rtol=1e-4, atol=1e-3, what=name)
 
 
+def test_column_split_of_a_partly_empty_last_round():
+    """4096 x 4608 are 16 x 18 = 288 tiles of 256 x 256 on 256 CUs, and no whole number of row bands makes a full round:
+    the 16 column bands of one full round (4096 columns) go to the 256 x 256 kernel, the 512 columns to their right to a
+    second launch (plan "a|b"), whose B, b_scale blocks and C start 4096 columns in.  int8: the integers of the single
+    launch everywhere and the oracle's on sampled rows (all columns, so both sides of the seam); fp8 block-scaled (the
+    right part must pick up b_scale at block row 32) and bf16: the oracle within tolerance on the same rows, and the
+    single launch everywhere."""
+    M, N, K = 4096, 4608, 2048
+    N1 = 4096
+    say("column split int8", M, N, K)
+    plan = Q.plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, M, N, K)
+    assert "|" in plan and "+" not in plan, plan
+    rng = np.random.default_rng(23)
+    qa = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    qb = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    da, db_ = dev(qa), dev(qb)
+    c = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+    Q.int8_mm(da, db_, scalar(1.0), scalar(1.0), c)
+    name = Q.last_config()
+    assert name == plan, (name, plan)
+    rows = np.concatenate([_sample(M, 20, 5), [0, M - 1]])
+    got = host(c)
+    assert np.array_equal(got[rows], R.gemm_i8_i32(qa[rows], qb)), name
+    cols = np.array([0, N1 - 1, N1, N1 + 127, N1 + 128, N - 1])
+    assert np.array_equal(got[:, cols], R.gemm_i8_i32(qa, qb[cols])), name
+    Q.set_option("row_split", 0)
+    c1 = torch.full((M, N), -8, dtype=torch.int32, device="cuda")
+    Q.int8_mm(da, db_, scalar(1.0), scalar(1.0), c1)
+    assert "|" not in Q.last_config() and "+" not in Q.last_config() and torch.equal(c, c1)
+    Q.set_option("row_split", 1)
+
+    say("column split fp8 block-scaled", M, N, K)
+    qa8, _ = R.quantize_fp8(R.fill_normal((M, K), 35))
+    qb8, _ = R.quantize_fp8(R.fill_normal((N, K), 36))
+    as_ = R.fill_uniform((M, K // 128), 37, 0.5, 2.0) / np.float32(448)
+    bs = R.fill_uniform((N // 128, K // 128), 38, 0.5, 2.0) / np.float32(448)
+    cb = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    Q.scaled_gemm(fp8_tensor(qa8), fp8_tensor(qb8), dev(as_), dev(bs), cb, M, N, K, Q.SCALE_BLOCK128)
+    name = Q.last_config()
+    assert "|" in name, name
+    ref = R.gemm_fp8_block(R.decode_fp8(qa8[rows]), R.decode_fp8(qb8), as_[rows], bs)
+    assert_close(host(cb)[rows], ref, what=name)
+    Q.set_option("row_split", 0)
+    cb1 = torch.zeros_like(cb)
+    Q.scaled_gemm(fp8_tensor(qa8), fp8_tensor(qb8), dev(as_), dev(bs), cb1, M, N, K, Q.SCALE_BLOCK128)
+    assert "|" not in Q.last_config()
+    assert torch.all((cb1.float() - cb.float()).abs() <= 2.0 ** -7 * cb.float().abs() + 1e-3)
+    Q.set_option("row_split", 1)
+
+    say("column split bf16, C with a leading dimension", M, N, K)
+    ha, hb = R.encode_bf16(R.fill_uniform((M, K), 43)), R.encode_bf16(R.fill_uniform((N, K), 44))
+    a16, b16 = dev(ha.view(np.int16)).view(torch.bfloat16), dev(hb.view(np.int16)).view(torch.bfloat16)
+    wide = torch.full((M, N + 64), -3.0, dtype=torch.float32, device="cuda")
+    c16 = wide[:, :N]
+    Q.gemm(a16, b16, c16, "nk")
+    name = Q.last_config()
+    assert "|" in name, name
+    assert_close(host(c16)[rows], R.gemm_f32acc(R.decode_bf16(ha[rows]), R.decode_bf16(hb)), rtol=1e-4, atol=1e-3, what=name)
+    assert torch.all(wide[:, N:] == -3.0)
+
+
 @pytest.mark.parametrize("shape,m_main,rest", [((4184, 4096, 2048), 4096, "skinny_64x64_k8"),      # 88 rows below one full round
                                                ((5000, 4096, 2048), 4096, "128x128")])            # single launch: 128 x 128 tiles
 def test_row_split_with_a_short_rest_and_against_smaller_tiles(shape, m_main, rest):
