@@ -350,6 +350,53 @@ def test_column_split_of_a_partly_empty_last_round():
     assert torch.all(wide[:, N:] == -3.0)
 
 
+def test_forced_row_and_column_splits_on_ragged_shapes_match_the_single_launch():
+    """Ragged M and N (not multiples of the tiles, of 128 or of 16), with the rows and then the columns of the full
+    rounds forced into a launch of their own wherever the geometry has such a split: the int32 results are those of
+    the single launch, element for element, and nothing is written beyond column N of a wider C.  fp8 with block
+    scales (ragged N: the last b_scale block row is partial) stays within a bf16 ulp of the single launch."""
+    rng = np.random.default_rng(2025)
+    shapes = [(4097, 4609, 640), (6000, 4500, 512), (3333, 9001, 384), (8200, 2300, 768), (5121, 5119, 400)]
+    seen = set()
+    try:
+        for (M, N, K) in shapes:
+            say("forced splits int8", M, N, K)
+            da = dev(rng.integers(-127, 128, (M, K), dtype=np.int8))
+            db_ = dev(rng.integers(-127, 128, (N, K), dtype=np.int8))
+            outs = {}
+            for mode in (0, 2, 3):
+                Q.set_option("row_split", mode)
+                wide = torch.full((M, N + 3), -9, dtype=torch.int32, device="cuda")
+                Q.int8_mm(da, db_, scalar(1.0), scalar(1.0), wide[:, :N])
+                name = Q.last_config()
+                assert torch.all(wide[:, N:] == -9), name
+                outs[mode] = wide[:, :N].clone()
+                seen.add("+" if "+" in name else ("|" if "|" in name else "one"))
+                assert mode != 0 or ("+" not in name and "|" not in name), name
+            assert torch.equal(outs[0], outs[2]) and torch.equal(outs[0], outs[3]), (M, N, K)
+        assert seen == {"+", "|", "one"}, seen
+
+        M, N, K = 4200, 4500, 640
+        say("forced splits fp8 block-scaled", M, N, K)
+        KB, NB = K // 128, (N + 127) // 128
+        qa8, _ = R.quantize_fp8(R.fill_normal((M, K), 61))
+        qb8, _ = R.quantize_fp8(R.fill_normal((N, K), 62))
+        as_ = dev(R.fill_uniform((M, KB), 63, 0.5, 2.0) / np.float32(448))
+        bs = dev(R.fill_uniform((NB, KB), 64, 0.5, 2.0) / np.float32(448))
+        a8, b8 = fp8_tensor(qa8), fp8_tensor(qb8)
+        outs = {}
+        for mode in (0, 2, 3):
+            Q.set_option("row_split", mode)
+            c = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+            Q.scaled_gemm(a8, b8, as_, bs, c, M, N, K, Q.SCALE_BLOCK128)
+            outs[mode] = (c.float(), Q.last_config())
+        assert "+" in outs[2][1] and "|" in outs[3][1], (outs[2][1], outs[3][1])
+        for mode in (2, 3):
+            assert torch.all((outs[mode][0] - outs[0][0]).abs() <= 2.0 ** -7 * outs[0][0].abs() + 1e-3), outs[mode][1]
+    finally:
+        Q.set_option("row_split", 1)
+
+
 @pytest.mark.parametrize("shape,m_main,rest", [((4184, 4096, 2048), 4096, "skinny_64x64_k8"),      # 88 rows below one full round
                                                ((5000, 4096, 2048), 4096, "128x128")])            # single launch: 128 x 128 tiles
 def test_row_split_with_a_short_rest_and_against_smaller_tiles(shape, m_main, rest):
