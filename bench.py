@@ -16,7 +16,7 @@ formula (:146-147).  That window is taken twice: as the first GPU work of the
 process (`cold_start`: the part was idle and its clock is still rising), and
 again behind the other configs and 300 more launches of the same GEMM, with no
 pause (`value`: the part under load).  See LOAD_MS in bench_util.py.  The tuning and
-probing modes (--shape, --vendor-sweep, --mid-sweep, --stream-sweep, --skinny-probe) live in
+probing modes (--shape, --vendor-sweep, --mid-sweep, --stream-sweep, --split-sweep, --skinny-probe) live in
 bench_modes.py.
 """
 import argparse
@@ -102,6 +102,9 @@ def main():
     ap.add_argument("--mid-sweep", action="store_true",
                     help="only time 160 ... 3072 rows against six weight shapes, this library and the vendor library from "
                          "replayed graphs, print one JSON line and exit")
+    ap.add_argument("--split-sweep", action="store_true",
+                    help="only time shapes with a partly empty last round of 256 x 256 tiles as one launch, split by rows, "
+                         "split by columns and as the planner has it, print one JSON line and exit")
     ap.add_argument("--shape", default="",
                     help="only run this library on one shape, e.g. fp8:2048x2048x8192 (fp8 | fp8block | int8 | int8f32 | bf16 | fp16), "
                          "--steps launches from a replayed graph; print one JSON line and exit")
@@ -139,6 +142,9 @@ def main():
         return 0
     if args.mid_sweep:
         print(json.dumps({"mid_sweep": bench_modes.mid_sweep(Q, torch, dev)}))
+        return 0
+    if args.split_sweep:
+        print(json.dumps({"split_sweep": bench_modes.split_sweep(Q, torch, dev)}))
         return 0
     if args.skinny_probe:
         print(json.dumps({"skinny_probe": bench_modes.skinny_probe(Q, torch, dev)}))

@@ -4,7 +4,7 @@ their commands."""
 import json
 import sys
 
-from bench_util import LOAD_MS, _graph_time, _quant_fp8, _quant_i8, _time_launches
+from bench_util import LOAD_MS, _graph_time, _quant_fp8, _quant_i8, _time_launches, _time_under_load
 
 # the shapes of the reference's report (TechniqueReport.md:117-121, 151-155) and a few that do not tile evenly
 SWEEP_SHAPES = [(1024, 512, 2048), (2048, 2048, 2048), (4096, 4096, 4096), (8192, 4096, 2048), (8192, 4096, 4096),
@@ -228,6 +228,50 @@ def mid_sweep(Q, torch, dev):
                     row["error"] = str(e)[:200]
                 rows.append(row)
                 print("[mid]", json.dumps(row), file=sys.stderr, flush=True)
+    return rows
+
+
+SPLIT_SHAPES = [(6144, 4608, 7168), (4096, 14336, 4096), (4096, 14336, 7168), (8192, 7168, 4096), (8192, 4608, 4096),
+                (8192, 4608, 2048), (4096, 4608, 4096), (2048, 28672, 4096), (6144, 6144, 6144), (5120, 5120, 5120),
+                (3072, 14336, 4096), (7000, 7168, 2048)]
+
+
+def split_sweep(Q, torch, dev):
+    """Shapes whose 256 x 256 tiles leave a partly empty last round of CUs: one launch, the rows of the full rounds and
+    the rows below as two launches, the same with columns, and what the planner takes (option "row_split" 0 / 2 / 3 /
+    1), fp8 per-matrix, fp8 with block scales and bf16; microseconds per launch, ten launches behind LOAD_MS of the
+    same call, the four settings in turn, twice; the vendor library beside them where it has the type."""
+    rows = []
+    for fam in ("fp8", "fp8block", "bf16"):
+        for (M, N, K) in SPLIT_SHAPES:
+            c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            vend = None
+            if fam == "bf16":
+                a = torch.randn(M, K, device=dev).bfloat16(); b = torch.randn(N, K, device=dev).bfloat16()
+                fn = lambda: Q.bf16_mm(a, b, c)
+                vend = lambda: torch.matmul(a, b.t(), out=c)
+            else:
+                a, sa = _quant_fp8(torch.randn(M, K, device=dev)); b, sb = _quant_fp8(torch.randn(N, K, device=dev))
+                if fam == "fp8":
+                    fn = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_PER_MATRIX)
+                    vend = lambda: torch._scaled_mm(a, b.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+                else:
+                    KB = (K + 127) // 128
+                    sa = (torch.rand(M, KB, device=dev) + 0.5) / 448; sb = (torch.rand((N + 127) // 128, KB, device=dev) + 0.5) / 448
+                    fn = lambda: Q.scaled_gemm(a, b, sa, sb, c, M, N, K, Q.SCALE_BLOCK128)
+            row = {"type": fam, "M": M, "N": N, "K": K}
+            try:
+                for rep in range(2):
+                    for key, mode in (("one_launch", 0), ("rows", 2), ("columns", 3), ("planner", 1)):
+                        Q.set_option("row_split", mode)
+                        row.setdefault(key + "_us", []).append(round(_time_under_load(fn, 10, 3) * 1e3, 1))
+                        row[key] = Q.last_config()
+                    if vend is not None:
+                        row.setdefault("vendor_us", []).append(round(_time_under_load(vend, 10, 3) * 1e3, 1))
+            finally:
+                Q.set_option("row_split", 1)
+            rows.append(row)
+            print("[split]", json.dumps(row), file=sys.stderr, flush=True)
     return rows
 
 

@@ -277,10 +277,14 @@ bool mfma_shape_ok(const NtProblem &q) {
 // plus 6 us around a round (2048 x 4096 x 4096 29.3 us, 1024 x 8192 x 8192 50.8, 1536 x 4096 x 4096 25.2,
 // 768 x 7168 x 2048 14.8; it wins where its tiles make one round of CUs and the 256 x 256 tiles would leave half of
 // them idle: 6 - 17 % over the two-stage 128 x 128 row there, with block scales up to 24 %).
-// 192 x 256 (8-wave solo schedule) for row counts whose 256-row tiles leave a round partly empty: 1.10 us a step in a
-// full round, 0.97 in a partly filled one (1.30 / 1.18 with block scales), 6 us around a round (3072 x 4096 x 4096 fp8
+// 192 x 256 (8-wave solo schedule) for row counts whose 256-row tiles leave a round partly empty: 1.03 us a step in a
+// full round, 0.97 in a partly filled one (1.27 / 1.18 with block scales), 6 us around a round (3072 x 4096 x 4096 fp8
 // 43.7 us against 47.5 on 192 tiles of 256 x 256, 2560 rows 37.7 against 42.8, 1536 x 7168 x 2048 23.3 against 26.8,
-// bf16 1152 x 8192 x 4096 64.6 against 78.3).
+// bf16 1152 x 8192 x 4096 64.6 against 78.3).  Full rounds refitted on 36 large shapes per type with every large row
+// forced (they had been priced at 1.10 / 1.30, 7 - 10 % above what was measured): shapes whose 192-row tiles make
+// whole rounds now run on them in one launch instead of a 256 x 256 launch and a rest (6144^3: 768 tiles, three
+// rounds; fp8 165.9 -> 163.7 us, block scales 206.9 -> 198.1, bf16 327.4 -> 318.5; over the 71 of 1440 grid shapes
+// whose plan changed the new plan is 3.0 % faster on average, at worst 1.6 % slower).
 // A K split adds 4 us and the partial planes at 3 TB/s.
 //
 // M <= 64 (bandwidth-bound, B is streamed once): the largest tile that still gives three quarters of the CUs a
@@ -303,7 +307,7 @@ struct TileModel {
 const TileModel kTileModels[] = {{256, 256, 1, 1.25, 1.25, 4.0, false, 1, 1.40, 1.40}, {128, 128, 2, 0.85, 0.66, 2.0, false, 2, 1.32, 1.04},
                                  {128, 128, 1, 0.43, 0.43, 4.5, true, 1, 0.50, 0.50},  {64, 128, 1, 0.52, 0.52, 1.5, false, 3, 1.21, 0.83},
                                  {64, 128, 1, 0.27, 0.27, 4.5, true, 1, 0.34, 0.34},   {128, 32, 1, 0.39, 0.39, 1.0, false, 2, 0.74, 0.60},
-                                 {256, 128, 1, 0.71, 0.58, 6.0, false, 1, 0.93, 0.76}, {192, 256, 1, 1.10, 0.97, 6.0, false, 1, 1.30, 1.18}};
+                                 {256, 128, 1, 0.71, 0.58, 6.0, false, 1, 0.93, 0.76}, {192, 256, 1, 1.03, 0.97, 6.0, false, 1, 1.27, 1.18}};
 // rows with two K groups: two sets of computing waves on a tile that otherwise has one (one workgroup per CU)
 bool is_kgroup_row(const Variant &v) { return v.kgroups == 2; }
 
