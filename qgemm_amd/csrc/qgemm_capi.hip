@@ -61,6 +61,7 @@ struct Context {
     long dbg_ptr = 0;           // measurement builds: device buffer for the kernels' time stamps (GemmArgs::dbg_cycles)
 #endif
     long as_groups = 1;         // 0: a_scale always one K block per copy on the rows with two K groups (see run_nt)
+    long small_tiles = 1;       // 0: 65 .. 256 rows never go to several row tiles of the skinny-M kernel in place of a K split
     long k_rot = -1;            // -1: rotated K start for at most 256 rows (see plan_nt), 0: never, n: steps per column tile
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long stagger_groups = 8;    // groups the workgroups of the first round start in
@@ -376,6 +377,37 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     // From 65 rows on: with two row tiles a workgroup pulls half of A (an L2 hit, but through its CU's load path) next
     // to twice the strip of B, 256 KiB instead of 320 KiB at 128 x 7168 x 2048, the smallest sum a tile of that area
     // has (config 5 at M = 128, B out of HBM: 8.9 -> 8.3 us; M = 64 stays on 32-column strips, 6.8 us).
+    // 65 .. 256 rows against few columns, 32 .. 48 K steps: tiles of 32 x 32, 64 x 32 or 64 x 64 on the skinny-M kernel,
+    // several over the rows, whichever fills at most one round of CUs with the least to move: a workgroup moves its rows
+    // of A and B at about 100 GB/s and all of them together about 12 TB/s (the row tiles of a strip share it in the
+    // L2s), 2.8 us around it.  That beats a taller tile with a K split across workgroups (a second launch of 4.5 us)
+    // and the 64 x 64 form where smaller tiles still fit a round.  Graph replays, us, one B / B in rotation through
+    // 600 MB, what the rules below took against this: 128 x 1024 x 4096 fp8 10.0 / 10.7 (128 x 32, four slices) ->
+    // 5.4 / 6.6 (32 x 32), 96 x 2048 x 4096 8.8 / 11.3 (64 x 64) -> 6.5 / 7.9, 128 x 2048 x 4096 8.8 / 11.8 -> 7.6 / 9.1
+    // (64 x 32), 130 x 1536 x 6144 12.8 / 13.7 -> 10.0 / 11.0; bf16 the same at the same bytes of K, block scales
+    // 128 x 2048 x 4096 10.5 / 13.0 -> 8.7 / 9.7.  From 56 K steps on the small tiles still win with B resident
+    // (160 x 2048 x 7168 13.5 -> 12.2) but lose with B streamed (14.9 -> 17.7: fewer, longer streams), so the K split
+    // stays there; block scales only up to 32 K steps (their fold makes the longer loops of the small tiles slower).
+    if (vi >= 0 && !kmaj && g_ctx.small_tiles && M > 64 && M <= 256 && ksteps >= 32 && ksteps <= (block ? 32u : 48u)) {
+        int best = -1;
+        double best_t = 0;
+        for (int i = 0; i < count; ++i) {
+            const Variant &v = tab[i];
+            if (v.kgroups != 8 || !((v.bm == 32 && v.bn == 32) || (v.bm == 64 && v.bn == 32) || (v.bm == 64 && v.bn == 64))) continue;
+            const size_t tiles = ((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
+            if (tiles > (size_t)cus) continue;
+            const double per_wg = (double)(v.bm + v.bn) * ksteps * 128.0;
+            const double t = std::max(per_wg / 100.0e3, tiles * per_wg / 12.0e6);
+            if (best < 0 || t < best_t) {
+                best = i;
+                best_t = t;
+            }
+        }
+        if (best >= 0) {
+            *nsplit_out = 1;
+            return best;
+        }
+    }
     if (vi >= 0 && !kmaj && M > 64 && ksteps >= 16 && ksteps <= 64) {
         const size_t t64 = ((M + 63) / 64) * ((N + 63) / 64);
         if (t64 <= (size_t)cus && (t64 >= 128 || (t64 >= 64 && ksteps <= 32)))
@@ -1079,6 +1111,7 @@ QGEMM_EXPORT int qgemm_set_option(const char *key, long value) {
     else if (!std::strcmp(key, "b_stream")) g_ctx.b_stream = value;
     else if (!std::strcmp(key, "k_rot")) g_ctx.k_rot = value;
     else if (!std::strcmp(key, "as_groups")) g_ctx.as_groups = value;
+    else if (!std::strcmp(key, "small_tiles")) g_ctx.small_tiles = value;
 #if QGEMM_DEBUG_BUILD
     else if (!std::strcmp(key, "dbg_ptr")) g_ctx.dbg_ptr = value;
 #endif

@@ -126,6 +126,19 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_BF16, 0, 0, 128, 7168, 2048) == "skinny_64x64_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 8192, 8192) == "skinny_64x64_k8"
     assert plan(Q.DT_BF16, 0, 0, 128, 8192, 8192) == "128x128_w2x2_k2_splitk4"
+    # 65 .. 256 rows against few columns, 32 .. 48 K steps: small tiles of the skinny-M kernel over several row tiles, whichever
+    # moves least in one round of CUs, instead of a taller tile with a K split (block scales: up to 32 K steps)
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 1024, 4096) == "skinny_32x32_k8"
+    assert plan(Q.DT_BF16, 0, 0, 128, 2048, 2048) == "skinny_64x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 96, 2048, 4096) == "skinny_32x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 130, 1536, 6144) == "skinny_64x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 2048, 7168) == "skinny_128x32_k8_splitk4"       # 56 steps: the split stays
+    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 130, 1536, 6144) != "skinny_64x32_k8"
+    Q.set_option("small_tiles", 0)
+    try:
+        assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 1024, 4096) == "skinny_128x32_k8_splitk4"
+    finally:
+        Q.set_option("small_tiles", 1)
     # ... but not with few K steps or where the estimate prefers wide tiles
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 7168, 512) == "128x32_w4x1_dma"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 8192, 1024) == "64x32_w4x1_dma"
