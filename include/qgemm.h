@@ -168,7 +168,7 @@ int qgemm_tile_map(uint32_t wg, uint32_t tiles_m, uint32_t tiles_n, uint32_t gro
  * qgemm_set_option(key, value): "force_split" (K slices, 0 = heuristic), "group_m", "kmajor", "stagger", "k_rot",
  *   "stagger_groups", "as_groups", "row_split" (0: one launch always; 1: the rows "a+b" or columns "a|b" of a partly
  *   empty last round of 256 x 256 tiles as a second launch where the estimate gains; 2 / 3: rows / columns wherever
- *   possible), "small_tiles" (0: 65 .. 256 rows against few columns keep a tall tile with a K split instead of several
+ *   possible), "small_tiles" (0: 17 .. 256 rows against few columns keep a tall tile with a K split instead of several
  *   row tiles of the skinny-M kernel), "c_plain" (0 / 1: non-temporal / ordinary stores for C; -1: the library's
  *   choice), "b_stream" (0 / 1: copies of B without / with the streaming hint; -1: the library's choice); "force_config" accepts only -1 (back to the heuristic).
  *   "k_rot": with at most 256 rows the workgroups of column tile i start their K loops 3 i steps in and wrap round

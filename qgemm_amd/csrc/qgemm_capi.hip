@@ -61,7 +61,7 @@ struct Context {
     long dbg_ptr = 0;           // measurement builds: device buffer for the kernels' time stamps (GemmArgs::dbg_cycles)
 #endif
     long as_groups = 1;         // 0: a_scale always one K block per copy on the rows with two K groups (see run_nt)
-    long small_tiles = 1;       // 0: 65 .. 256 rows never go to several row tiles of the skinny-M kernel in place of a K split
+    long small_tiles = 1;       // 0: 17 .. 256 rows never go to several row tiles of the skinny-M kernel in place of a K split
     long k_rot = -1;            // -1: rotated K start for at most 256 rows (see plan_nt), 0: never, n: steps per column tile
     long stagger = -1;          // -1: staggered start where it pays (4-byte C, three or more rounds), else microseconds per group
     long stagger_groups = 8;    // groups the workgroups of the first round start in
@@ -377,10 +377,11 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     // From 65 rows on: with two row tiles a workgroup pulls half of A (an L2 hit, but through its CU's load path) next
     // to twice the strip of B, 256 KiB instead of 320 KiB at 128 x 7168 x 2048, the smallest sum a tile of that area
     // has (config 5 at M = 128, B out of HBM: 8.9 -> 8.3 us; M = 64 stays on 32-column strips, 6.8 us).
-    // 65 .. 256 rows against few columns, 32 .. 48 K steps: tiles of 32 x 32, 64 x 32 or 64 x 64 on the skinny-M kernel,
+    // 17 .. 256 rows against few columns, 32 .. 48 K steps: tiles of 16 x 32, 32 x 32, 64 x 32 or 64 x 64 on the skinny-M kernel,
     // several over the rows, whichever fills at most one round of CUs with the least to move: a workgroup moves its rows
-    // of A and B at about 100 GB/s and all of them together about 12 TB/s (the row tiles of a strip share it in the
-    // L2s), 2.8 us around it.  That beats a taller tile with a K split across workgroups (a second launch of 4.5 us)
+    // of A at about 100 GB/s (L2 hits) and its strip of B at about 45 GB/s (out of memory), all of them together about
+    // 12 TB/s (the row tiles of a strip share it in the L2s); constants fitted on 90 shapes x 4 tiles x (one B, B in
+    // rotation through 600 MB).  That beats a taller tile with a K split across workgroups (a second launch of 4.5 us)
     // and the 64 x 64 form where smaller tiles still fit a round.  Graph replays, us, one B / B in rotation through
     // 600 MB, what the rules below took against this: 128 x 1024 x 4096 fp8 10.0 / 10.7 (128 x 32, four slices) ->
     // 5.4 / 6.6 (32 x 32), 96 x 2048 x 4096 8.8 / 11.3 (64 x 64) -> 6.5 / 7.9, 128 x 2048 x 4096 8.8 / 11.8 -> 7.6 / 9.1
@@ -388,21 +389,26 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     // 128 x 2048 x 4096 10.5 / 13.0 -> 8.7 / 9.7.  From 56 K steps on the small tiles still win with B resident
     // (160 x 2048 x 7168 13.5 -> 12.2) but lose with B streamed (14.9 -> 17.7: fewer, longer streams), so the K split
     // stays there; block scales only up to 32 K steps (their fold makes the longer loops of the small tiles slower).
-    if (vi >= 0 && !kmaj && g_ctx.small_tiles && M > 64 && M <= 256 && ksteps >= 32 && ksteps <= (block ? 32u : 48u)) {
+    // 24 .. 256 rows x 1024 .. 7168 columns x 4 and 6 KiB of K, fp8, 90 shapes: 13 % less time with B resident, 9.5 % with B
+    // streamed, two shapes more than 3 % slower (7 % at worst); 64 x 1024 x 4096 fp8 7.7 / 8.5 (64 x 32, four slices) ->
+    // 4.7 / 5.6 (16 x 32).  A smaller tile has to be estimated 3 % ahead of a larger one.
+    if (vi >= 0 && !kmaj && g_ctx.small_tiles && M > 16 && M <= 256 && ksteps >= 32 && ksteps <= (block ? 32u : 48u)) {
         int best = -1;
         double best_t = 0;
-        for (int i = 0; i < count; ++i) {
-            const Variant &v = tab[i];
-            if (v.kgroups != 8 || !((v.bm == 32 && v.bn == 32) || (v.bm == 64 && v.bn == 32) || (v.bm == 64 && v.bn == 64))) continue;
-            const size_t tiles = ((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
-            if (tiles > (size_t)cus) continue;
-            const double per_wg = (double)(v.bm + v.bn) * ksteps * 128.0;
-            const double t = std::max(per_wg / 100.0e3, tiles * per_wg / 12.0e6);
-            if (best < 0 || t < best_t) {
-                best = i;
-                best_t = t;
+        static const int kSmall[4][2] = {{64, 64}, {64, 32}, {32, 32}, {16, 32}};       // (a smaller tile has to be 3 % ahead)
+        for (const auto &bt : kSmall)
+            for (int i = 0; i < count; ++i) {
+                const Variant &v = tab[i];
+                if (v.kgroups != 8 || v.bm != bt[0] || v.bn != bt[1]) continue;
+                const size_t tiles = ((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
+                if (tiles > (size_t)cus) continue;
+                const double kb = ksteps * 128.0;
+                const double t = std::max(v.bm * kb / 100.0e3 + v.bn * kb / 45.0e3, tiles * (v.bm + v.bn) * kb / 12.0e6);
+                if (best < 0 || t < 0.97 * best_t) {
+                    best = i;
+                    best_t = t;
+                }
             }
-        }
         if (best >= 0) {
             *nsplit_out = 1;
             return best;

@@ -126,14 +126,17 @@ def test_plan_names_the_kernel_without_a_device():
     assert plan(Q.DT_BF16, 0, 0, 128, 7168, 2048) == "skinny_64x64_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 8192, 8192) == "skinny_64x64_k8"
     assert plan(Q.DT_BF16, 0, 0, 128, 8192, 8192) == "128x128_w2x2_k2_splitk4"
-    # 65 .. 256 rows against few columns, 32 .. 48 K steps: small tiles of the skinny-M kernel over several row tiles, whichever
+    # 17 .. 256 rows against few columns, 32 .. 48 K steps: small tiles of the skinny-M kernel over several row tiles, whichever
     # moves least in one round of CUs, instead of a taller tile with a K split (block scales: up to 32 K steps)
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 1024, 4096) == "skinny_32x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 1024, 4096) == "skinny_32x32_k8"                # (was 128 x 32 with four K slices)
     assert plan(Q.DT_BF16, 0, 0, 128, 2048, 2048) == "skinny_64x32_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 96, 2048, 4096) == "skinny_32x32_k8"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 130, 1536, 6144) == "skinny_64x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 130, 1536, 6144) == "skinny_32x32_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 1024, 4096) == "skinny_16x32_k8"                 # (was 64 x 32 with four K slices)
+    assert plan(Q.DT_BF16, 0, 0, 48, 2048, 2048) == "skinny_16x32_k8"
+    assert plan(Q.DT_BF16, 0, 0, 64, 7168, 2048) == "skinny_64x32_k8"                                    # (wide: one row tile, as before)
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 2048, 7168) == "skinny_128x32_k8_splitk4"       # 56 steps: the split stays
-    assert plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 130, 1536, 6144) != "skinny_64x32_k8"
+    assert "splitk" in plan(Q.DT_F8E4M3, Q.SCALE_BLOCK128, 0, 130, 1536, 6144)                            # (block scales: only up to 32 steps)
     Q.set_option("small_tiles", 0)
     try:
         assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 1024, 4096) == "skinny_128x32_k8_splitk4"
