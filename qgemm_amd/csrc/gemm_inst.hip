@@ -130,6 +130,8 @@ static std::vector<Variant> build_table() {
         add(skinny_row<4>("skinny_64x32_k8"));
         add(skinny_row<8>("skinny_128x32_k8"));
         add(skinny_row<4, 4>("skinny_64x64_k8"));
+        add(skinny_row<1, 1>("skinny_16x16_k8"));
+        add(skinny_row<2, 1>("skinny_32x16_k8"));
     }
     // 256 x 128 on the solo schedule with four computing waves (128 x 64 wave tiles, one per SIMD) and four copying
     // waves (GemmCfg::COPYW): block scales and K-major operands on a large tile; its twin for K-contiguous a_scale

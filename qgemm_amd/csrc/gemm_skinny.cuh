@@ -46,7 +46,10 @@ struct SkinnyCfg {
     static constexpr int RING_BYTES = SLOTS * 1024;
     static constexpr int LDS_BYTES = NW * RING_BYTES;       // the rings; afterwards one partial sum (1 KiB per tile) per wave
     static_assert(TM == 1 || TM == 2 || TM == 4 || TM == 8, "the programs below are written for these tile heights");
-    static_assert(TN == 2 || (TN == 4 && TM == 4), "64-column strips: the 64 x 64 tile");
+    static_assert(TN == 2 || (TN == 4 && TM == 4) || (TN == 1 && TM <= 2), "64-column strips: the 64 x 64 tile; 16-column strips: up to 32 rows");
+    // TN = 1 (16-column strips, up to 32 rows; with 64 rows they were level with 32-column strips and a K split or behind): twice the strips of the 32-column rows, for few columns against a long K,
+    // where 32-column strips leave half of the CUs idle and a K split across workgroups costs a second launch.
+    static constexpr bool ALL_AT_ONCE = 2 * (SA + SB) <= SLOTS;      // both steps of a round fit the ring together
     static_assert(TM * TN * 1024 <= RING_BYTES, "a wave's partial sums fit its ring");
 };
 
@@ -244,7 +247,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
     };
 
     // ---- one round = steps k and k + 8 of this wave.  Ring programs by tile height (slots per step: A 2 TM, B 4):
-    //   TM <= 2  (at most 16 slots): everything at once.                 B0 B1 A0 A1
+    //   TM <= 2, or 16-column strips (at most 20 slots): everything at once.   B0 B1 A0 A1
     //   TM == 4  (24 slots):  A0 B0 B1 A1[0..4)  | A0 drained ->  A1[4..8)
     //   TM == 8  (40 slots):  A0[0..12) B0 B1    | A0[0..12) drained -> A0[12..16) A1[0..8) | B0 B1 A0[12..16) drained
     //                         -> A1[8..16)
@@ -260,7 +263,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
             copy_a(k, 0, 8, 0);
             copy_b(k, 8);
             copy_b_part(k + C::NW, 0, 4, 16);
-        } else if constexpr (C::TM <= 2) {
+        } else if constexpr (C::ALL_AT_ONCE) {
             copy_b(k, 0);
             copy_b(k + C::NW, SB);
             copy_a(k, 0, SA, 2 * SB);
@@ -300,7 +303,7 @@ __global__ void __launch_bounds__(C::THREADS) gemm_skinny_kernel(const GemmArgs 
             drain_a(1, 0, 2, 4);
             wait_landed<0>();
             drain_a(1, 2, 2, 8);
-        } else if constexpr (C::TM <= 2) {
+        } else if constexpr (C::ALL_AT_ONCE) {
             wait_landed<SA>();
             drain_b(0, 0);
             drain_b(1, SB);

@@ -425,6 +425,23 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     }
     if (vi < 0 || kmaj || M > 128) return vi;
     const size_t strips = (N + 31) / 32;
+    // Up to 32 rows against so few columns that 32-column strips leave half of the CUs idle, 32 .. 112 K steps: strips of
+    // 16 columns, one workgroup each and no K split across workgroups (which costs a second launch).  Graph replays, us,
+    // one B / B in rotation through 600 MB, fp8 (bf16 the same at the same bytes of K): 16 x 4096 x 14336 14.7 / 15.8
+    // (32-column strips, two slices) -> 12.6 / 13.0 (vendor library 12.7 / 14.7), 16 x 4096 x 8192 11.5 / 12.1 -> 9.4 / 9.0,
+    // 16 x 2048 x 8192 7.2 / 9.6 -> 5.6 / 7.7, 32 x 4096 x 14336 16.2 / 18.1 -> 15.8 / 16.6; from 128 K steps on the split is
+    // ahead (16 x 2048 x 16384 10.2 / 11.0 against 12.2 / 13.2), and with 64 rows the two are level or the split ahead.
+    // With fewer than 192 such strips (N < 3072) only up to 16 rows and 64 K steps: beyond that the streams are too few
+    // and too long, and the split is 4 - 50 % ahead with B streamed (32 x 1024 x 14336 9.5 against 14.7 us).  Not with block
+    // scales (3 - 30 % slower throughout).
+    const size_t strips16 = (N + 15) / 16;
+    if (g_ctx.small_tiles && !block && M <= 32 && ksteps >= 32 && ksteps <= 112 && strips * 2 <= (size_t)cus && strips16 <= (size_t)cus &&
+        (strips16 >= 192 || (M <= 16 && ksteps <= 64)))
+        for (int i = 0; i < count; ++i)
+            if (tab[i].kgroups == 8 && tab[i].bn == 16 && (size_t)tab[i].bm >= M) {     // (rows of the table in ascending height)
+                *nsplit_out = 1;
+                return i;
+            }
     // 33 .. 64 rows against so many columns that the 32-column strips need a second round of CUs while 64-column
     // strips fit in one: the 64 x 64 form (half the strips, each row of A fetched half as often).  B out of HBM:
     // 64 x 14336 x 4096 bf16 34.3 -> 26.7 us, fp8 20.4 -> 17.0; 48 rows 33.4 -> 27.4 and 19.4 -> 16.5.

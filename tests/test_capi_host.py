@@ -115,8 +115,12 @@ def test_plan_names_the_kernel_without_a_device():
         assert plan(Q.DT_I8, Q.SCALE_PER_MATRIX, 0, m, 7168, 2048) == name
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 24, 4096, 4096) == "skinny_32x32_k8"
     # ... with a K split across workgroups on top where the strips leave half of the CUs idle and K is long
-    assert plan(Q.DT_BF16, 0, 0, 24, 4096, 4096) == "skinny_32x32_k8_splitk2"
-    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 4096, 14336) == "skinny_16x32_k8_splitk2"
+    assert plan(Q.DT_BF16, 0, 0, 24, 4096, 16384) == "skinny_32x32_k8_splitk2"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 4096, 28672) == "skinny_16x32_k8_splitk2"
+    # ... or, up to 32 rows and 32 .. 112 K steps, strips of 16 columns, twice as many and no K split
+    assert plan(Q.DT_BF16, 0, 0, 24, 4096, 4096) == "skinny_32x16_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 4096, 14336) == "skinny_16x16_k8"
+    assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 2048, 16384) == "skinny_16x32_k8_splitk4"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 2048, 8192) == "skinny_64x32_k8_splitk4"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 16, 8192, 8192) == "skinny_16x32_k8"
     # 33 .. 64 rows whose 32-column strips need a second round of CUs: 64-column strips; 65 .. 128 rows whose strips
