@@ -442,10 +442,12 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
                 *nsplit_out = 1;
                 return i;
             }
-    // 33 .. 64 rows against so many columns that the 32-column strips need a second round of CUs while 64-column
+    // 17 .. 64 rows against so many columns that the 32-column strips need a second round of CUs while 64-column
     // strips fit in one: the 64 x 64 form (half the strips, each row of A fetched half as often).  B out of HBM:
-    // 64 x 14336 x 4096 bf16 34.3 -> 26.7 us, fp8 20.4 -> 17.0; 48 rows 33.4 -> 27.4 and 19.4 -> 16.5.
-    if (M > 32 && M <= 64 && ksteps >= 16 && strips > (size_t)cus && (N + 63) / 64 <= (size_t)cus)
+    // 64 x 14336 x 4096 bf16 34.3 -> 26.7 us, fp8 20.4 -> 17.0; 48 rows 33.4 -> 27.4 and 19.4 -> 16.5; 32 rows bf16
+    // 26.4 -> 23.5, 32 x 14336 x 8192 49.7 -> 41.2, 24 x 11008 x 4096 24.4 -> 22.5, 32 x 12288 x 2048 fp8 10.4 -> 9.1
+    // (up to 16 rows the two are level).
+    if (M > 16 && M <= 64 && ksteps >= 16 && strips > (size_t)cus && (N + 63) / 64 <= (size_t)cus)
         for (int i = 0; i < count; ++i)
             if (tab[i].kgroups == 8 && tab[i].bm == 64 && tab[i].bn == 64) {
                 *nsplit_out = 1;

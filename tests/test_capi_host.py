@@ -126,6 +126,8 @@ def test_plan_names_the_kernel_without_a_device():
     # 33 .. 64 rows whose 32-column strips need a second round of CUs: 64-column strips; 65 .. 128 rows whose strips
     # fit one round and K is not long: the skinny-M kernel rather than what the estimate (of resident operands) likes
     assert plan(Q.DT_BF16, 0, 0, 64, 14336, 4096) == "skinny_64x64_k8"
+    assert plan(Q.DT_BF16, 0, 0, 32, 14336, 4096) == "skinny_64x64_k8"          # (from 17 rows on; 16 rows stay on 32-column strips)
+    assert plan(Q.DT_BF16, 0, 0, 16, 14336, 4096) == "skinny_16x32_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 64, 8192, 8192) == "skinny_64x32_k8"
     assert plan(Q.DT_BF16, 0, 0, 128, 7168, 2048) == "skinny_64x64_k8"
     assert plan(Q.DT_F8E4M3, Q.SCALE_PER_MATRIX, 0, 128, 8192, 8192) == "skinny_64x64_k8"
