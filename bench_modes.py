@@ -154,7 +154,10 @@ def one_shape(Q, torch, dev, spec, launches):
 STREAM_SHAPES = [(1, 8192, 8192), (16, 4096, 4096), (16, 4096, 14336), (64, 4096, 14336), (16, 8192, 8192), (64, 8192, 8192),
                  (128, 8192, 8192), (16, 14336, 4096), (32, 14336, 4096), (64, 14336, 4096), (128, 14336, 4096),
                  (16, 28672, 8192), (64, 28672, 8192), (128, 28672, 4096), (32, 8192, 28672), (16, 7168, 2048),
-                 (64, 7168, 2048), (128, 7168, 2048)]
+                 (64, 7168, 2048), (128, 7168, 2048),
+                 # few columns (grouped-query K / V projections, small experts): where the tile choice fills the CUs with
+                 # small tiles or narrow strips instead of a K split across workgroups
+                 (16, 1024, 8192), (64, 1024, 8192), (64, 1024, 4096), (128, 1024, 4096), (128, 2048, 4096), (256, 2048, 4096)]
 
 
 def stream_sweep(Q, torch, dev):

@@ -416,7 +416,10 @@ int choose_variant(const Variant *tab, int count, size_t M, size_t N, size_t kst
     }
     if (vi >= 0 && !kmaj && M > 64 && ksteps >= 16 && ksteps <= 64) {
         const size_t t64 = ((M + 63) / 64) * ((N + 63) / 64);
-        if (t64 <= (size_t)cus && (t64 >= 128 || (t64 >= 64 && ksteps <= 32)))
+        // (with more than 48 K steps and weights streamed out of memory, half a round of such tiles is behind a wider tile
+        // with a K split, which has twice the streams: 256 x 2048 x 8192 fp8 18.3 against 16.1 us, 13.5 against 13.8 with
+        // B resident; from 160 tiles on the 64 x 64 form is ahead either way)
+        if (t64 <= (size_t)cus && ((t64 >= 128 && (ksteps <= 48 || t64 >= 160)) || (t64 >= 64 && ksteps <= 32)))
             for (int i = 0; i < count; ++i)
                 if (tab[i].kgroups == 8 && tab[i].bm == 64 && tab[i].bn == 64) {
                     *nsplit_out = 1;
